@@ -1,0 +1,379 @@
+#!/usr/bin/env python3
+"""Benchmark of the causal conv1d hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu]
+
+Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill shape
+(bf16, batch 8, dim 5376, seqlen 2048, channel-last, width 4, bias, SiLU, seq_idx with
+1-4 packed sub-sequences per row), inputs resident in HBM before the timed region.
+
+  value / unit ..... algorithmic bytes moved per second by that forward (GB/s); the
+                     algorithmic bytes count every input element read once and every
+                     output element written once (x, out, seq_idx, weight, bias)
+  roofline ......... the same bytes over the average kernel time measured with HIP events
+                     around the timed launches, against the 8 TB/s HBM3E peak
+  cpu_baseline ..... the PyTorch oracle (F.conv1d per packed sub-sequence) timed on this
+                     host's cores on the same inputs
+  others ........... µs per call and GB/s of the remaining shapes: decode-step update
+                     (linear and circular state), backward, varlen state gather, and the
+                     forward width/dtype sweep; "rotated" figures cycle through enough
+                     distinct buffer sets to exceed the 256 MB Infinity Cache
+
+The timed loops call the extension entry points directly with pre-allocated outputs, the
+way the reference's own benchmark does (tests/benchmark_determinism_kernels.py:72).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG_DIR = os.path.join(ROOT, "causal-conv1d_amd")
+for _p in (ROOT, PKG_DIR):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+INFINITY_CACHE_BYTES = 256 * 1024 * 1024
+
+
+# --------------------------------------------------------------------------- workloads
+def _gen(seed):
+    import torch
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def make_weights(dim, width, seed, w_dtype=None):
+    import torch
+    g = _gen(1000 + seed)
+    w = torch.rand(dim, width, generator=g) - 0.5
+    b = torch.rand(dim, generator=g) - 0.5
+    if w_dtype is not None:
+        w, b = w.to(w_dtype), b.to(w_dtype)
+    return w, b
+
+
+def make_seq_idx(batch, seqlen, seed, max_segments=4):
+    """Per row: 1..max_segments packed sub-sequences with random boundaries, ids 0..n-1."""
+    import torch
+    g = _gen(2000 + seed)
+    rows = []
+    for _ in range(batch):
+        n = int(torch.randint(1, max_segments + 1, (1,), generator=g))
+        n = min(n, seqlen)
+        cuts = torch.randperm(seqlen - 1, generator=g)[: n - 1].sort().values + 1 if seqlen > 1 else torch.tensor([], dtype=torch.long)
+        bounds = [0] + cuts.tolist() + [seqlen]
+        rows.append(torch.cat([torch.full((bounds[i + 1] - bounds[i],), i, dtype=torch.int32)
+                               for i in range(len(bounds) - 1)]))
+    return torch.stack(rows)
+
+
+def make_x(batch, dim, seqlen, dtype, channel_last, seed):
+    """N(0,1) tensor of logical shape (batch, dim, seqlen) in the requested memory layout."""
+    import torch
+    g = _gen(seed)
+    if channel_last:
+        return torch.randn(batch, seqlen, dim, generator=g).to(dtype).transpose(1, 2)
+    return torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+
+
+def config_c1():
+    import torch
+    w, b = make_weights(64, 4, 1)
+    return dict(x=make_x(2, 64, 512, torch.float32, False, 1), weight=w, bias=b)
+
+
+def config_c2(batch=8, dim=5376, seqlen=2048):
+    import torch
+    w, b = make_weights(dim, 4, 2)
+    return dict(x=make_x(batch, dim, seqlen, torch.bfloat16, True, 2), weight=w, bias=b,
+                seq_idx=make_seq_idx(batch, seqlen, 2))
+
+
+def config_c3(circular, batch=256, dim=5376, seed=3):
+    import torch
+    w, b = make_weights(dim, 4, 3)
+    state_len = 8 if circular else 3
+    g = _gen(3000 + seed)
+    cfg = dict(x=make_x(batch, dim, 1, torch.bfloat16, True, seed), weight=w, bias=b,
+               conv_state=make_x(batch, dim, state_len, torch.bfloat16, True, seed + 50))
+    if circular:
+        cfg["cache_seqlens"] = torch.randint(0, 1000, (batch,), generator=g, dtype=torch.int32)
+    return cfg
+
+
+def config_c4(batch=4, dim=4096, seqlen=8192):
+    import torch
+    w, b = make_weights(dim, 4, 4)
+    return dict(x=make_x(batch, dim, seqlen, torch.float16, False, 4), weight=w, bias=b,
+                dout=make_x(batch, dim, seqlen, torch.float16, False, 41),
+                initial_states=make_x(batch, dim, 3, torch.float16, True, 42),
+                dfinal_states=make_x(batch, dim, 3, torch.float16, False, 43))
+
+
+def config_c5a(total=65536, n_seq=64, dim=5376):
+    import torch
+    g = _gen(5)
+    lens = torch.randint(16, 2048, (n_seq,), generator=g).double()
+    lens = torch.clamp((lens / lens.sum() * total).floor().long(), min=3)
+    lens[-1] += total - int(lens.sum())
+    assert int(lens.sum()) == total and int(lens.min()) >= 3
+    cu = torch.nn.functional.pad(lens.cumsum(0), (1, 0)).to(torch.int32)
+    x = torch.randn(total, dim, generator=g).to(torch.bfloat16)
+    return dict(x=x, cu_seqlens=cu, state_len=3)
+
+
+def config_c5b(width, dtype, channel_last, batch=4, dim=2048, seqlen=4096):
+    w, b = make_weights(dim, width, 50 + width)
+    return dict(x=make_x(batch, dim, seqlen, dtype, channel_last, 50 + width), weight=w, bias=b)
+
+
+def nbytes(*tensors):
+    return sum(t.numel() * t.element_size() for t in tensors if t is not None)
+
+
+# ------------------------------------------------------------------------------ timing
+def time_gpu(fn, steps, warmup):
+    """Average µs per call of fn(i) over `steps` calls after `warmup`, by HIP events on the
+    current stream, with the device idle on both sides."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) * 1e3 / steps, wall * 1e6 / steps
+
+
+def to_dev(cfg, dev):
+    import torch
+    return {k: (v.to(dev) if isinstance(v, torch.Tensor) else v) for k, v in cfg.items()}
+
+
+def clone_sets(cfg, bytes_per_set, max_sets=64):
+    """Enough independent copies of the device tensors to exceed the Infinity Cache."""
+    import torch
+    n = min(max_sets, max(2, math.ceil(2 * INFINITY_CACHE_BYTES / max(1, bytes_per_set))))
+    def cp(v):
+        if not isinstance(v, torch.Tensor):
+            return v
+        if v.dim() == 3 and v.stride(1) == 1 and v.stride(2) > 1:      # keep channel-last
+            return v.transpose(1, 2).clone().transpose(1, 2)
+        return v.clone()
+    return [{k: cp(v) for k, v in cfg.items()} for _ in range(n)]
+
+
+def gbs(n_bytes, us):
+    return n_bytes / us * 1e-3 if us > 0 else 0.0
+
+
+# ---------------------------------------------------------------------- the other shapes
+def bench_others(ext, dev, steps, warmup):
+    import torch
+    res = {}
+
+    def record(name, us, n_bytes, extra=None):
+        res[name] = {"us": round(us, 3), "GBps": round(gbs(n_bytes, us), 1),
+                     "frac_of_hbm_peak": round(gbs(n_bytes, us) / HBM_PEAK_GBS, 4),
+                     "algorithmic_bytes": int(n_bytes)}
+        if extra:
+            res[name].update(extra)
+
+    # C3: decode-step update, linear and circular.
+    for circular in (False, True):
+        name = "update_circular_s8" if circular else "update_linear_s3"
+        cfg = to_dev(config_c3(circular), dev)
+        x, st = cfg["x"], cfg["conv_state"]
+        n_bytes = nbytes(x, x, cfg["weight"], cfg["bias"])
+        if circular:
+            n_bytes += 3 * nbytes(x) + nbytes(x) + nbytes(cfg["cache_seqlens"])   # window read + 1 row written
+        else:
+            n_bytes += 2 * nbytes(st)
+        out = torch.empty_like(x)
+        cs = cfg.get("cache_seqlens")
+        us, wall = time_gpu(lambda i: ext.causal_conv1d_update(x, st, cfg["weight"], cfg["bias"], out, True, cs, None),
+                            steps, warmup)
+        sets = clone_sets(cfg, nbytes(x, st, x))
+        outs = [torch.empty_like(s["x"]) for s in sets]
+        def rot(i):
+            s = sets[i % len(sets)]
+            ext.causal_conv1d_update(s["x"], s["conv_state"], s["weight"], s["bias"], outs[i % len(sets)], True,
+                                     s.get("cache_seqlens"), None)
+        us_rot, _ = time_gpu(rot, steps, warmup)
+        record(name, us, n_bytes, {"us_rotated": round(us_rot, 3),
+                                   "GBps_rotated": round(gbs(n_bytes, us_rot), 1),
+                                   "frac_of_hbm_peak_rotated": round(gbs(n_bytes, us_rot) / HBM_PEAK_GBS, 4),
+                                   "rotated_sets": len(sets), "us_wall_per_call": round(wall, 2)})
+        del sets, outs
+
+    # C4: backward, fp16 channel-first with initial states and dfinal.
+    cfg = to_dev(config_c4(), dev)
+    x = cfg["x"]
+    dx = torch.empty_like(x)
+    dw = torch.zeros(x.shape[1], 4, device=dev, dtype=torch.float32)
+    db = torch.zeros(x.shape[1], device=dev, dtype=torch.float32)
+    dinit = torch.empty(x.shape[0], 3, x.shape[1], device=dev, dtype=x.dtype).transpose(1, 2)
+    n_bytes = nbytes(x, cfg["dout"], dx, cfg["initial_states"], cfg["dfinal_states"], dinit,
+                     cfg["weight"], cfg["bias"], dw, db)
+    us, _ = time_gpu(lambda i: ext.causal_conv1d_bwd(x, cfg["weight"], cfg["bias"], cfg["dout"], None,
+                                                     cfg["initial_states"], cfg["dfinal_states"], dx, dw, db, dinit, True),
+                     max(10, steps // 4), max(3, warmup // 4))
+    record("bwd_c4_fp16_channelfirst", us, n_bytes)
+    del cfg, x, dx
+
+    # Backward, channel-last at the prefill shape (bf16, seq_idx).
+    cfg = to_dev(config_c2(), dev)
+    x = cfg["x"]
+    dout = to_dev(dict(d=make_x(8, 5376, 2048, torch.bfloat16, True, 21)), dev)["d"]
+    dx = torch.empty_like(x)
+    dw = torch.zeros(x.shape[1], 4, device=dev, dtype=torch.float32)
+    db = torch.zeros(x.shape[1], device=dev, dtype=torch.float32)
+    n_bytes = nbytes(x, dout, dx, cfg["seq_idx"], cfg["weight"], cfg["bias"], dw, db)
+    us, _ = time_gpu(lambda i: ext.causal_conv1d_bwd(x, cfg["weight"], cfg["bias"], dout, cfg["seq_idx"],
+                                                     None, None, dx, dw, db, None, True),
+                     max(10, steps // 4), max(3, warmup // 4))
+    record("bwd_prefill_bf16_channellast_seqidx", us, n_bytes)
+    del cfg, x, dx, dout
+
+    # C5a: varlen state gather.
+    cfg = to_dev(config_c5a(), dev)
+    states = torch.empty(64, 3, 5376, device=dev, dtype=torch.bfloat16).transpose(1, 2)
+    n_bytes = 2 * nbytes(states) + nbytes(cfg["cu_seqlens"])
+    us, _ = time_gpu(lambda i: ext.causal_conv1d_varlen_states(cfg["x"], cfg["cu_seqlens"], states, 3), steps, warmup)
+    record("varlen_states_c5a", us, n_bytes)
+    del cfg
+
+    # C5b: forward sweep over width x dtype x layout.
+    for dtype, dn in ((torch.float32, "fp32"), (torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+        for layout in (False, True):
+            for width in (2, 3, 4):
+                cfg = to_dev(config_c5b(width, dtype, layout), dev)
+                x = cfg["x"]
+                out = torch.empty_like(x)
+                n_bytes = nbytes(x, out, cfg["weight"], cfg["bias"])
+                us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(x, cfg["weight"], cfg["bias"], None, None, out, None, True),
+                                 max(20, steps // 2), max(5, warmup // 2))
+                record("fwd_sweep_%s_%s_w%d" % (dn, "channellast" if layout else "channelfirst", width), us, n_bytes)
+    return res
+
+
+# ------------------------------------------------------------------------ CPU baseline
+def cpu_baseline(cfg_cpu, n_bytes):
+    """The PyTorch oracle on the host, same inputs, whole C2 workload per repetition."""
+    import torch
+    from oracle import causal_conv1d_oracle as orc
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    x, w, b, seq = cfg_cpu["x"], cfg_cpu["weight"], cfg_cpu["bias"], cfg_cpu["seq_idx"]
+    with torch.no_grad():
+        orc.fwd_seq_idx(x, w, b, seq, activation="silu")           # warm-up
+        times = []
+        t_end = time.perf_counter() + 20.0
+        while len(times) < 5 and (len(times) < 2 or time.perf_counter() < t_end):
+            t0 = time.perf_counter()
+            orc.fwd_seq_idx(x, w, b, seq, activation="silu")
+            times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(n_bytes / med * 1e-9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "us_per_call": round(med * 1e6, 1),
+            "sample": "the full prefill workload (8 x 5376 x 2048 bf16 + seq_idx), median of %d calls "
+                      "of the PyTorch F.conv1d oracle after one warm-up" % len(times)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
+    ap.add_argument("--rows", type=int, default=0, help="override rows per lane run (sweeps)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
+                 "(the operator needs no cross-GPU communication; run one process per GPU on disjoint batches)" % args.gpus)
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the benchmark has no CPU fallback")
+    import causal_conv1d_cuda as ext          # fails loudly if the extension was not built
+    dev = torch.device("cuda:0")
+
+    cfg_cpu = config_c2()
+    cfg = to_dev(cfg_cpu, dev)
+    x, w, b, seq = cfg["x"], cfg["weight"], cfg["bias"], cfg["seq_idx"]
+    out = torch.empty_like(x)
+    n_bytes = nbytes(x, out, seq, w, b)
+    if args.rows:
+        import ctypes
+        lib = ctypes.CDLL(os.path.join(PKG_DIR, "libcc1d.so"))
+        lib.cc1d_set_tunable(b"fwd_cl_rows", ctypes.c_int32(args.rows))
+
+    def step(i):
+        ext.causal_conv1d_fwd(x, w, b, seq, None, out, None, True)
+
+    us, wall_us = time_gpu(step, args.steps, args.warmup)
+
+    # Parity of what was just timed, against the oracle on a slice small enough to be quick.
+    from oracle import causal_conv1d_oracle as orc
+    ref = orc.fwd_seq_idx(cfg_cpu["x"][:1], cfg_cpu["weight"], cfg_cpu["bias"], cfg_cpu["seq_idx"][:1], activation="silu")
+    got = out[:1].float().cpu()
+    err = (got - ref.float()).abs()
+    parity_ok = bool(torch.all(err <= 5e-2 + 1e-2 * ref.float().abs()))
+
+    # End-to-end through the public Python API (allocation + op dispatch included).
+    from causal_conv1d import causal_conv1d_fn
+    with torch.no_grad():
+        _, api_wall = time_gpu(lambda i: causal_conv1d_fn(x, w, b, seq_idx=seq, activation="silu"),
+                               max(20, args.steps // 4), max(5, args.warmup // 4))
+
+    line = {
+        "metric": "fwd/bwd/update µs per call + achieved HBM GB/s (% of MI355X peak)",
+        "value": round(gbs(n_bytes, us), 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us * 1e-3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "Mamba-2 2.7B prefill forward: bf16 x (8, 5376, 2048) channel-last, width 4, "
+                               "bias, SiLU, int32 seq_idx with 1-4 packed sub-sequences per row",
+                   "algorithmic_bytes": int(n_bytes), "us_per_call": round(us, 3),
+                   "us_per_call_python_api_wall": round(api_wall, 2),
+                   "parity_vs_oracle_ok": parity_ok, "max_abs_err": float(err.max())},
+        "roofline": {"bound": "hbm", "achieved": round(gbs(n_bytes, us), 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs(n_bytes, us) / HBM_PEAK_GBS, 4), "traffic": None},
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "fwd_channellast_prefill_traffic.txt")
+    if os.path.exists(traffic_file):
+        for ln in open(traffic_file):
+            if ln.startswith("traffic_bytes_per_launch:"):
+                line["roofline"]["traffic"] = int(float(ln.split(":")[1]))
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(cfg_cpu, n_bytes)
+    del cfg, x, out
+    if not args.no_others:
+        try:
+            line["others"] = bench_others(ext, dev, args.steps, args.warmup)
+        except Exception as e:                                      # keep the headline line intact
+            line["others"] = {"error": repr(e)}
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

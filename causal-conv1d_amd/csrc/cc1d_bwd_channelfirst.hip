@@ -1,0 +1,349 @@
+// Channel-first backward for gfx950.  Takes over causal_conv1d_bwd_kernel and its
+// launcher (csrc/causal_conv1d_bwd.cu:53-293 of the reference).  Formulas as in the
+// channel-last backward; initial_states / dfinal_states / dinitial_states are supported
+// for this layout too (the reference refuses them, csrc/causal_conv1d.cpp:349,364).
+//
+// Design.  A wavefront owns one channel and a contiguous slice of that channel's
+// (batch x segment) items, so its dweight/dbias partial sums live in registers across
+// all of them and are reduced over the 64 lanes once, at the very end.  With one slice
+// per channel (the usual case, dim >= 4096) the sums go straight to dweight/dbias and no
+// workspace exists; otherwise each slice stores W+1 floats and the shared second-stage
+// kernel adds the slices in a fixed order.  Either way the result is bit-reproducible.
+//
+// Inside an item the wave walks DOWN the row, 64 sixteen-byte vectors per step:
+//  * the x halo on the left comes from the previous lane (DPP shift); lane 0 takes it
+//    from lane 63 of the already prefetched next (lower) step;
+//  * g = dout * act'(z) is needed W-1 positions to the right for dx: from the next lane
+//    (DPP shift), lane 63 takes it from lane 0 of the previous (higher) step.
+// Only an item's first and last step fall back to a few wave-uniform element loads.
+// Rows of x, dout and dx may sit on different 16-byte grids; lanes follow x's grid and
+// the other tensors use vectors when they share it, elements otherwise.
+#include "cc1d_device.hpp"
+#include "cc1d_internal.hpp"
+
+namespace cc1d {
+namespace {
+
+struct BwdCfGeom {
+    int32_t vecs_per_seg;     // multiple of 64
+    int32_t n_segs;           // segments per row
+    int32_t n_items;          // batch * n_segs
+    int32_t n_parts;          // slices of the item list per channel
+    int32_t items_per_part;
+};
+
+template <int DT>
+struct alignas(16) RawT {
+    typename Elem<DT>::type v[Elem<DT>::kVec];
+};
+
+template <int DT, int W>
+struct RowCtx {
+    const cc1d_bwd_params &p;
+    int b, c;
+    int64_t xrow, drow;
+    float wv[W];
+    float bias_v;
+    bool silu_on;
+
+    // xpad[t] for t < L, raw bits
+    __device__ __forceinline__ typename Elem<DT>::type x_raw_at(int t) const {
+        using T = typename Elem<DT>::type;
+        if (t >= 0) return ld_raw<DT>(p.x, xrow + t);
+        if (p.initial_states != nullptr && t >= -(W - 1))
+            return ld_raw<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
+                                                    (int64_t)c * p.init_stride_c +
+                                                    (int64_t)(t + W - 1) * p.init_stride_l);
+        return T(0.f);
+    }
+    // xpad[t] for t < L (fp32)
+    __device__ __forceinline__ float x_at(int t) const {
+        if (t >= 0) return ld_elem<DT>(p.x, xrow + t);
+        if (p.initial_states != nullptr && t >= -(W - 1))
+            return ld_elem<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
+                                                     (int64_t)c * p.init_stride_c +
+                                                     (int64_t)(t + W - 1) * p.init_stride_l);
+        return 0.f;
+    }
+    // g[t] recomputed from memory with the same operation order as the vector path.
+    __device__ __forceinline__ float g_at(int t) const {
+        if (t < 0 || t >= p.seqlen) return 0.f;
+        float gv = ld_elem<DT>(p.dout, drow + t);
+        if (silu_on) {
+            float z = bias_v;
+#pragma unroll
+            for (int w = 0; w < W; ++w) z = fmaf(wv[w], x_at(t - (W - 1) + w), z);
+            gv *= silu_grad<Elem<DT>::kPreciseAct>(z);
+        }
+        return gv;
+    }
+};
+
+template <int DT, int W>
+__global__ void __launch_bounds__(kBlock)
+bwd_channelfirst_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__restrict__ ws) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    constexpr int VEC = E::kVec;
+    constexpr bool PRECISE = E::kPreciseAct;
+
+    const uint32_t wid = (blockIdx.x * (uint32_t)kBlock + threadIdx.x) / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    if (wid >= (uint32_t)p.dim * (uint32_t)g.n_parts) return;     // whole wave leaves together
+    const int part = (int)(wid % (uint32_t)g.n_parts);
+    const int c = (int)(wid / (uint32_t)g.n_parts);
+    const int L = p.seqlen;
+
+    RowCtx<DT, W> rc{p};
+    rc.c = c;
+    rc.silu_on = p.silu != 0;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+        rc.wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
+    rc.bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+
+    float dW[W], dB = 0.f;
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = 0.f;
+
+    const int item_begin = part * g.items_per_part;
+    int item_end = item_begin + g.items_per_part;
+    if (item_end > g.n_items) item_end = g.n_items;
+
+    for (int item = item_begin; item < item_end; ++item) {
+        const int seg = item % g.n_segs;
+        const int b = item / g.n_segs;
+        rc.b = b;
+        rc.xrow = (int64_t)b * p.x_stride_b + (int64_t)c * p.x_stride_c;
+        rc.drow = (int64_t)b * p.dout_stride_b + (int64_t)c * p.dout_stride_c;
+        const int64_t dxrow = (int64_t)b * p.dx_stride_b + (int64_t)c * p.dx_stride_c;
+        const int mis = (int)((reinterpret_cast<uintptr_t>(reinterpret_cast<const T *>(p.x) + rc.xrow) / sizeof(T)) % VEC);
+        const int mis_d = (int)((reinterpret_cast<uintptr_t>(reinterpret_cast<const T *>(p.dout) + rc.drow) / sizeof(T)) % VEC);
+        const int mis_dx = (int)((reinterpret_cast<uintptr_t>(reinterpret_cast<T *>(p.dx) + dxrow) / sizeof(T)) % VEC);
+        const bool dout_same = mis_d == mis, dx_same = mis_dx == mis;
+
+        const int n_vecs = (L + mis + VEC - 1) / VEC;
+        const int j_begin = seg * g.vecs_per_seg;
+        int j_end = j_begin + g.vecs_per_seg;
+        if (j_end > n_vecs) j_end = n_vecs;
+
+        if (j_begin < j_end) {
+            // Raw 16-byte vectors on x's grid; positions outside [0, L) read as zero
+            // (or initial_states for x), element by element where a vector does not fit.
+            auto load_x = [&](int j) -> u32x4 {
+                const int tf = j * VEC - mis;
+                if (tf >= 0 && tf + VEC <= L) return ld_vec_nt<DT>(p.x, rc.xrow + tf);
+                RawT<DT> r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) r.v[e] = (tf + e < L) ? rc.x_raw_at(tf + e) : T(0.f);
+                return bitcast<u32x4>(r);
+            };
+            auto load_d = [&](int j) -> u32x4 {
+                const int tf = j * VEC - mis;
+                if (dout_same && tf >= 0 && tf + VEC <= L) return ld_vec_nt<DT>(p.dout, rc.drow + tf);
+                RawT<DT> r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    r.v[e] = (tf + e >= 0 && tf + e < L) ? ld_raw<DT>(p.dout, rc.drow + tf + e) : T(0.f);
+                return bitcast<u32x4>(r);
+            };
+
+            // g just right of the item (positions of the following segment, or beyond L).
+            float carry_g[W - 1];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) carry_g[i] = rc.g_at(j_end * VEC - mis + i);
+
+            // Two steps of loads stay in flight: r1 is the next (lower) step, r2 the one after.
+            const int n_steps = (j_end - j_begin + kWave - 1) / kWave;
+            const u32x4 zero4 = {0u, 0u, 0u, 0u};
+            u32x4 r1x = load_x(j_begin + (n_steps - 1) * kWave + lane);
+            u32x4 r1d = load_d(j_begin + (n_steps - 1) * kWave + lane);
+            u32x4 r2x = zero4, r2d = zero4;
+            if (n_steps > 1) {
+                r2x = load_x(j_begin + (n_steps - 2) * kWave + lane);
+                r2d = load_d(j_begin + (n_steps - 2) * kWave + lane);
+            }
+
+            for (int s = n_steps - 1; s >= 0; --s) {
+                const int j0 = j_begin + s * kWave;
+                float xf[VEC], gf[VEC];
+                E::unpack(r1x, xf);
+                E::unpack(r1d, gf);
+                r1x = r2x; r1d = r2d;
+                if (s >= 2) {
+                    r2x = load_x(j0 - 2 * kWave + lane);
+                    r2d = load_d(j0 - 2 * kWave + lane);
+                }
+
+                // x just left of this step: lane 63 of the next (lower) step, which was
+                // requested a whole step ago; memory only at the item's lowest step.
+                float carry_x[W - 1];
+                if (s > 0) {
+                    float lower[VEC];
+                    E::unpack(r1x, lower);
+#pragma unroll
+                    for (int i = 0; i < W - 1; ++i) carry_x[i] = read_lane(lower[VEC - (W - 1) + i], kWave - 1);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < W - 1; ++i) carry_x[i] = rc.x_at(j0 * VEC - mis - (W - 1) + i);
+                }
+
+                // xx[i] = xpad at position tf-(W-1)+i
+                float xx[VEC + W - 1];
+#pragma unroll
+                for (int i = 0; i < W - 1; ++i) xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry_x[i]);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xf[e];
+
+                if (rc.silu_on) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        float z = rc.bias_v;
+#pragma unroll
+                        for (int w = 0; w < W; ++w) z = fmaf(rc.wv[w], xx[e + w], z);
+                        gf[e] *= silu_grad<PRECISE>(z);
+                    }
+                }
+
+                // gg[i] = g at position tf+i, i in [0, VEC+W-1)
+                float gg[VEC + W - 1];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) gg[e] = gf[e];
+#pragma unroll
+                for (int i = 0; i < W - 1; ++i) {
+                    gg[VEC + i] = from_next_lane(gf[i], carry_g[i]);
+                    carry_g[i] = read_lane(gf[i], 0);
+                }
+
+                const int j = j0 + lane;
+                const int tf = j * VEC - mis;
+                float dxv[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float a = 0.f;
+#pragma unroll
+                    for (int k = 0; k < W; ++k) a = fmaf(rc.wv[W - 1 - k], gg[e + k], a);
+                    dxv[e] = a;
+                }
+                if (p.dfinal_states != nullptr && tf + VEC > L - (W - 1)) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const int t = tf + e;
+                        if (t >= 0 && t >= L - (W - 1) && t < L)
+                            dxv[e] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
+                                                                      (int64_t)c * p.dfinal_stride_c +
+                                                                      (int64_t)(t - (L - (W - 1))) * p.dfinal_stride_l);
+                    }
+                }
+                if (j < j_end) {
+                    if (dx_same && tf >= 0 && tf + VEC <= L) {
+                        st_vec_nt<DT>(p.dx, dxrow + tf, E::pack(dxv));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            if (tf + e >= 0 && tf + e < L) st_elem<DT>(p.dx, dxrow + tf + e, dxv[e]);
+                    }
+                }
+
+                // Partial sums.  Lanes past j_end and positions outside [0, L) hold g == 0.
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    dB += gf[e];
+#pragma unroll
+                    for (int w = 0; w < W; ++w) dW[w] = fmaf(gf[e], xx[e + w], dW[w]);
+                }
+            }
+        }
+
+        // dinitial_states[b, c, i], i = lane < W-1, by the wave that owns the row's start.
+        if (p.dinitial_states != nullptr && seg == 0 && lane < W - 1) {
+            const int pp = lane - (W - 1);
+            float a = 0.f;
+#pragma unroll
+            for (int k = 0; k < W; ++k) a = fmaf(rc.wv[W - 1 - k], rc.g_at(pp + k), a);
+            if (p.dfinal_states != nullptr && lane >= L)
+                a += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
+                                                     (int64_t)c * p.dfinal_stride_c +
+                                                     (int64_t)(lane - L) * p.dfinal_stride_l);
+            st_elem<DT>(p.dinitial_states, (int64_t)b * p.dinit_stride_b + (int64_t)c * p.dinit_stride_c +
+                                               (int64_t)lane * p.dinit_stride_l, a);
+        }
+    }
+
+    // One fixed-order reduction over the wave, then a single writer.
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = wave_sum(dW[w]);
+    dB = wave_sum(dB);
+    if (lane == 0) {
+        if (g.n_parts == 1) {
+#pragma unroll
+            for (int w = 0; w < W; ++w)
+                p.dweight[(int64_t)c * p.dw_stride_c + (int64_t)w * p.dw_stride_w] += dW[w];
+            if (p.dbias != nullptr) p.dbias[c] += dB;
+        } else {
+            float *dst = ws + (int64_t)part * (W + 1) * p.dim + c;
+#pragma unroll
+            for (int w = 0; w < W; ++w) dst[(int64_t)w * p.dim] = dW[w];
+            dst[(int64_t)W * p.dim] = dB;
+        }
+    }
+}
+
+BwdCfGeom make_geom(const cc1d_bwd_params &p) {
+    const int vec = vec_elems(p.x_dtype);
+    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
+    const int64_t max_steps = (max_vecs + kWave - 1) / kWave;     // 64-vector steps per row
+    // About 16 waves on each of 256 CUs when the problem allows it.
+    int64_t parts = tunables().bwd_cf_parts > 0 ? tunables().bwd_cf_parts
+                                                : (4096 + p.dim - 1) / p.dim;
+    const int64_t max_parts = (int64_t)p.batch * max_steps;
+    if (parts > max_parts) parts = max_parts;
+    if (parts < 1) parts = 1;
+    // Split rows into segments only if there are fewer rows per channel than slices.
+    int64_t n_segs = (parts + p.batch - 1) / p.batch;
+    int64_t vps = (max_steps + n_segs - 1) / n_segs * kWave;
+    n_segs = (max_vecs + vps - 1) / vps;
+    BwdCfGeom g;
+    g.vecs_per_seg = (int32_t)vps;
+    g.n_segs = (int32_t)n_segs;
+    g.n_items = (int32_t)(p.batch * n_segs);
+    g.items_per_part = (int32_t)((g.n_items + parts - 1) / parts);
+    g.n_parts = (g.n_items + g.items_per_part - 1) / g.items_per_part;
+    return g;
+}
+
+template <int DT>
+int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStream_t stream) {
+    const int64_t waves = (int64_t)p.dim * g.n_parts;
+    if (waves >= ((int64_t)1 << 25)) return CC1D_ERR_TOO_LARGE;
+    const uint32_t blocks = (uint32_t)((waves + (kBlock / kWave) - 1) / (kBlock / kWave));
+    switch (p.width) {
+        case 2: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        case 3: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        default: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+    }
+    return launch_status();
+}
+
+}  // namespace
+
+size_t bwd_channelfirst_workspace_bytes(const cc1d_bwd_params &p) {
+    const BwdCfGeom g = make_geom(p);
+    if (g.n_parts == 1) return 0;
+    return (size_t)g.n_parts * (p.width + 1) * (size_t)p.dim * sizeof(float);
+}
+
+int launch_bwd_channelfirst(const cc1d_bwd_params &p, void *workspace, hipStream_t stream) {
+    const BwdCfGeom g = make_geom(p);
+    float *ws = static_cast<float *>(workspace);
+    int st;
+    switch (p.x_dtype) {
+        case CC1D_F32: st = launch_dtype<CC1D_F32>(p, g, ws, stream); break;
+        case CC1D_F16: st = launch_dtype<CC1D_F16>(p, g, ws, stream); break;
+        default: st = launch_dtype<CC1D_BF16>(p, g, ws, stream); break;
+    }
+    if (st != CC1D_OK || g.n_parts == 1) return st;
+    return launch_bwd_finalize(ws, g.n_parts, p, stream);
+}
+
+}  // namespace cc1d

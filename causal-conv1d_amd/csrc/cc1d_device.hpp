@@ -1,0 +1,254 @@
+// Device-side building blocks shared by every kernel of the library: element type
+// traits, 16-byte vector access, wave64 lane shifts (DPP), SiLU and per-lane weight
+// loading.  Written for gfx950 only (64-lane wavefronts, v_cvt_pk_bf16_f32).
+//
+// Takes over the roles of csrc/causal_conv1d_common.h:46-98 (BytesToType, Allreduce)
+// and csrc/static_switch.h:16-25 of the reference, with a different design: one lane
+// always owns one 16-byte vector, and cross-lane traffic is a DPP shift by one lane.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cc1d.h"
+
+namespace cc1d {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;  // 4 wavefronts per workgroup
+
+template <typename To, typename From>
+__device__ __forceinline__ To bitcast(const From &v) {
+    return __builtin_bit_cast(To, v);
+}
+
+// ---------------------------------------------------------------------------------
+// Element traits.  kVec elements make one 16-byte vector.
+// ---------------------------------------------------------------------------------
+template <int DT> struct Elem;
+
+template <> struct Elem<CC1D_F32> {
+    using type = float;
+    static constexpr int kVec = 4;
+    static constexpr int kBytes = 4;
+    // fp32 I/O is held to atol 1e-5 against the PyTorch reference, so SiLU uses the
+    // correctly rounded expf and a true division.
+    static constexpr bool kPreciseAct = true;
+    static __device__ __forceinline__ float to_float(float v) { return v; }
+    static __device__ __forceinline__ float from_float(float v) { return v; }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float (&f)[4]) {
+        f[0] = bitcast<float>(r.x); f[1] = bitcast<float>(r.y);
+        f[2] = bitcast<float>(r.z); f[3] = bitcast<float>(r.w);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[4]) {
+        u32x4 r;
+        r.x = bitcast<uint32_t>(f[0]); r.y = bitcast<uint32_t>(f[1]);
+        r.z = bitcast<uint32_t>(f[2]); r.w = bitcast<uint32_t>(f[3]);
+        return r;
+    }
+};
+
+template <> struct Elem<CC1D_F16> {
+    using type = _Float16;
+    static constexpr int kVec = 8;
+    static constexpr int kBytes = 2;
+    static constexpr bool kPreciseAct = false;
+    static __device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
+    static __device__ __forceinline__ _Float16 from_float(float v) { return (_Float16)v; }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float (&f)[8]) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f16x2 h = bitcast<f16x2>(w[i]);
+            f[2 * i] = (float)h.x;
+            f[2 * i + 1] = (float)h.y;
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f16x2 h;
+            h.x = (_Float16)f[2 * i];
+            h.y = (_Float16)f[2 * i + 1];
+            w[i] = bitcast<uint32_t>(h);
+        }
+        u32x4 r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+        return r;
+    }
+};
+
+template <> struct Elem<CC1D_BF16> {
+    using type = __bf16;
+    static constexpr int kVec = 8;
+    static constexpr int kBytes = 2;
+    static constexpr bool kPreciseAct = false;
+    static __device__ __forceinline__ float to_float(__bf16 v) { return (float)v; }
+    static __device__ __forceinline__ __bf16 from_float(float v) { return (__bf16)v; }
+    static __device__ __forceinline__ void unpack(const u32x4 &r, float (&f)[8]) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = bitcast<float>(w[i] << 16);
+            f[2 * i + 1] = bitcast<float>(w[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bf16x2 h;                       // round-to-nearest-even: v_cvt_pk_bf16_f32
+            h.x = (__bf16)f[2 * i];
+            h.y = (__bf16)f[2 * i + 1];
+            w[i] = bitcast<uint32_t>(h);
+        }
+        u32x4 r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+        return r;
+    }
+};
+
+// ---------------------------------------------------------------------------------
+// Global memory access.  Offsets are element offsets, always 64-bit.
+// ---------------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ u32x4 ld_vec(const void *base, int64_t elem_off) {
+    using T = typename Elem<DT>::type;
+    return *reinterpret_cast<const u32x4 *>(reinterpret_cast<const T *>(base) + elem_off);
+}
+template <int DT>
+__device__ __forceinline__ void st_vec(void *base, int64_t elem_off, const u32x4 &v) {
+    using T = typename Elem<DT>::type;
+    *reinterpret_cast<u32x4 *>(reinterpret_cast<T *>(base) + elem_off) = v;
+}
+// Streaming variants: data that is touched once should not displace the L2 contents.
+template <int DT>
+__device__ __forceinline__ u32x4 ld_vec_nt(const void *base, int64_t elem_off) {
+    using T = typename Elem<DT>::type;
+    return __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4 *>(reinterpret_cast<const T *>(base) + elem_off));
+}
+template <int DT>
+__device__ __forceinline__ void st_vec_nt(void *base, int64_t elem_off, const u32x4 &v) {
+    using T = typename Elem<DT>::type;
+    __builtin_nontemporal_store(
+        v, reinterpret_cast<u32x4 *>(reinterpret_cast<T *>(base) + elem_off));
+}
+template <int DT>
+__device__ __forceinline__ float ld_elem(const void *base, int64_t elem_off) {
+    using T = typename Elem<DT>::type;
+    return Elem<DT>::to_float(reinterpret_cast<const T *>(base)[elem_off]);
+}
+template <int DT>
+__device__ __forceinline__ void st_elem(void *base, int64_t elem_off, float v) {
+    using T = typename Elem<DT>::type;
+    reinterpret_cast<T *>(base)[elem_off] = Elem<DT>::from_float(v);
+}
+// Bit-preserving element copy (state shifts and gathers must be exact).
+template <int DT>
+__device__ __forceinline__ typename Elem<DT>::type ld_raw(const void *base, int64_t elem_off) {
+    using T = typename Elem<DT>::type;
+    return reinterpret_cast<const T *>(base)[elem_off];
+}
+template <int DT>
+__device__ __forceinline__ void st_raw(void *base, int64_t elem_off, typename Elem<DT>::type v) {
+    using T = typename Elem<DT>::type;
+    reinterpret_cast<T *>(base)[elem_off] = v;
+}
+
+// Weight / bias element of runtime type `w_dtype`, as fp32.
+__device__ __forceinline__ float ld_weight(const void *base, int w_dtype, int64_t elem_off) {
+    if (w_dtype == CC1D_F32) return reinterpret_cast<const float *>(base)[elem_off];
+    if (w_dtype == CC1D_F16) return (float)reinterpret_cast<const _Float16 *>(base)[elem_off];
+    return (float)reinterpret_cast<const __bf16 *>(base)[elem_off];
+}
+
+// Weights and bias of NCH consecutive channels starting at c0 into registers.
+// contiguous_f32 is a host-checked promise: fp32, strides (W, 1), 16-byte aligned base;
+// then NCH*W consecutive floats are fetched as 16-byte vectors.
+template <int W, int NCH>
+__device__ __forceinline__ void load_weights(const void *weight, const void *bias, int w_dtype,
+                                             int64_t stride_c, int64_t stride_w,
+                                             bool contiguous_f32, int c0,
+                                             float (&wv)[NCH][W], float (&bv)[NCH]) {
+    static_assert((NCH * W) % 4 == 0, "NCH*W floats must be whole 16-byte vectors");
+    if (contiguous_f32) {
+        float flat[NCH * W];
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(
+            reinterpret_cast<const float *>(weight) + (int64_t)c0 * W);
+#pragma unroll
+        for (int i = 0; i < NCH * W / 4; ++i) {
+            u32x4 r = src[i];
+            flat[4 * i] = bitcast<float>(r.x); flat[4 * i + 1] = bitcast<float>(r.y);
+            flat[4 * i + 2] = bitcast<float>(r.z); flat[4 * i + 3] = bitcast<float>(r.w);
+        }
+#pragma unroll
+        for (int j = 0; j < NCH; ++j)
+#pragma unroll
+            for (int w = 0; w < W; ++w) wv[j][w] = flat[j * W + w];
+    } else {
+#pragma unroll
+        for (int j = 0; j < NCH; ++j)
+#pragma unroll
+            for (int w = 0; w < W; ++w)
+                wv[j][w] = ld_weight(weight, w_dtype, (int64_t)(c0 + j) * stride_c + w * stride_w);
+    }
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+        bv[j] = bias == nullptr ? 0.f : ld_weight(bias, w_dtype, c0 + j);
+}
+
+// ---------------------------------------------------------------------------------
+// Wave64 lane shifts through DPP (no LDS, no memory).  All 64 lanes must be active.
+//   from_prev_lane: lane i receives lane i-1's value, lane 0 receives `lane0_fill`.
+//   from_next_lane: lane i receives lane i+1's value, lane 63 receives `lane63_fill`.
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ float from_prev_lane(float v, float lane0_fill) {
+    return bitcast<float>(__builtin_amdgcn_update_dpp(
+        bitcast<int>(lane0_fill), bitcast<int>(v), 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float from_next_lane(float v, float lane63_fill) {
+    return bitcast<float>(__builtin_amdgcn_update_dpp(
+        bitcast<int>(lane63_fill), bitcast<int>(v), 0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return bitcast<float>(__builtin_amdgcn_readlane(bitcast<int>(v), lane));
+}
+// Sum over the 64 lanes of a wave in a fixed butterfly order (deterministic).
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------
+// Activation.
+// ---------------------------------------------------------------------------------
+template <bool PRECISE>
+__device__ __forceinline__ float sigmoid(float z) {
+    if (PRECISE) {
+        return 1.0f / (1.0f + expf(-z));
+    } else {
+        // v_exp_f32 + v_rcp_f32: about 2 ulp, far inside the 16-bit output rounding.
+        return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.4426950408889634f));
+    }
+}
+template <bool PRECISE>
+__device__ __forceinline__ float silu(float z) {
+    if (PRECISE) {
+        return z / (1.0f + expf(-z));
+    } else {
+        return z * sigmoid<false>(z);
+    }
+}
+// d silu(z) / dz = s (1 + z (1 - s)),  s = sigmoid(z)  (csrc/causal_conv1d_bwd.cu:168-170)
+template <bool PRECISE>
+__device__ __forceinline__ float silu_grad(float z) {
+    const float s = sigmoid<PRECISE>(z);
+    return s * (1.0f + z * (1.0f - s));
+}
+
+}  // namespace cc1d

@@ -1,0 +1,195 @@
+// Channel-first forward for gfx950: x is (batch, dim, seqlen) with unit stride along
+// seqlen.  Takes over causal_conv1d_fwd_kernel and its launcher
+// (csrc/causal_conv1d_fwd.cu:46-170 of the reference).
+//
+// Design.  One wavefront owns one segment of one (batch, channel) row and walks it in
+// steps of 64 sixteen-byte vectors (1 KiB).  A lane's W-1 left neighbours come from the
+// previous lane through a DPP wave shift; lane 0 takes them from lane 63 of the wave's
+// previous step (v_readlane), so only a segment's very first step touches memory for
+// its halo.  There is no LDS and no barrier, and rows are spread over
+// (row x segment) waves instead of one serial loop per row.
+//
+// Rows need not be 16-byte aligned or a multiple of the vector length: lanes are laid
+// out on the row's own 16-byte grid (`mis` = elements between that grid and the row
+// start), vectors that stick out of [0, seqlen) are accessed element by element, and
+// the same holds for `out` when its rows sit on a different grid than x's.
+// initial_states / final_states are supported (the reference refuses them for this
+// layout, csrc/causal_conv1d.cpp:213,228).
+#include "cc1d_device.hpp"
+#include "cc1d_internal.hpp"
+
+namespace cc1d {
+namespace {
+
+struct FwdCfGeom {
+    int32_t vecs_per_seg;     // multiple of 64
+    int32_t n_segs;           // segments per row
+    uint32_t total_waves;     // batch * dim * n_segs
+};
+
+// Element t of the zero/initial-state padded row (fp32), for any t < L.
+template <int DT, int W>
+__device__ __forceinline__ float padded_elem(const cc1d_fwd_params &p, int64_t xrow, int b, int c,
+                                             int t) {
+    if (t >= 0) return ld_elem<DT>(p.x, xrow + t);
+    if (p.initial_states != nullptr && t >= -(W - 1))
+        return ld_elem<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
+                                                 (int64_t)c * p.init_stride_c +
+                                                 (int64_t)(t + W - 1) * p.init_stride_l);
+    return 0.f;
+}
+
+template <int DT, int W>
+__global__ void __launch_bounds__(kBlock)
+fwd_channelfirst_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
+    using E = Elem<DT>;
+    constexpr int VEC = E::kVec;
+    constexpr bool PRECISE = E::kPreciseAct;
+
+    const uint32_t wid = (blockIdx.x * (uint32_t)kBlock + threadIdx.x) / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    if (wid >= g.total_waves) return;                 // whole wave leaves together
+    const int seg = (int)(wid % (uint32_t)g.n_segs);
+    const uint32_t row = wid / (uint32_t)g.n_segs;
+    const int c = (int)(row % (uint32_t)p.dim);
+    const int b = (int)(row / (uint32_t)p.dim);
+    const int L = p.seqlen;
+    const bool silu_on = p.silu != 0;
+
+    const int64_t xrow = (int64_t)b * p.x_stride_b + (int64_t)c * p.x_stride_c;
+    const int64_t orow = (int64_t)b * p.out_stride_b + (int64_t)c * p.out_stride_c;
+    using T = typename E::type;
+    const int mis = (int)((reinterpret_cast<uintptr_t>(reinterpret_cast<const T *>(p.x) + xrow) /
+                           sizeof(T)) % VEC);
+    const int mis_o = (int)((reinterpret_cast<uintptr_t>(reinterpret_cast<T *>(p.out) + orow) /
+                             sizeof(T)) % VEC);
+    const bool out_same_grid = mis_o == mis;
+
+    const int n_vecs = (L + mis + VEC - 1) / VEC;     // vectors of this row on its grid
+    const int j_begin = seg * g.vecs_per_seg;
+    int j_end = j_begin + g.vecs_per_seg;
+    if (j_end > n_vecs) j_end = n_vecs;
+
+    if (j_begin < j_end) {
+        float wv[W], bias_v;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+            wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
+        bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+
+        // Halo of the segment's first vector, wave-uniform.
+        float carry[W - 1];
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i)
+            carry[i] = padded_elem<DT, W>(p, xrow, b, c, j_begin * VEC - mis - (W - 1) + i);
+
+        auto load_step = [&](int j, float (&xf)[VEC]) {
+            const int tf = j * VEC - mis;
+            if (tf >= 0 && tf + VEC <= L) {
+                E::unpack(ld_vec_nt<DT>(p.x, xrow + tf), xf);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    xf[e] = (tf + e < L) ? padded_elem<DT, W>(p, xrow, b, c, tf + e) : 0.f;
+            }
+        };
+
+        float nxt[VEC];
+        load_step(j_begin + lane, nxt);
+        for (int j0 = j_begin; j0 < j_end; j0 += kWave) {
+            float xf[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xf[e] = nxt[e];
+            if (j0 + kWave < j_end) load_step(j0 + kWave + lane, nxt);   // prefetch
+
+            // xx[i] = padded x at position tf - (W-1) + i
+            float xx[VEC + W - 1];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) {
+                xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry[i]);
+                carry[i] = read_lane(xf[VEC - (W - 1) + i], kWave - 1);
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xf[e];
+
+            float acc[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float a = bias_v;
+#pragma unroll
+                for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
+                acc[e] = silu_on ? silu<PRECISE>(a) : a;
+            }
+
+            const int j = j0 + lane;
+            const int tf = j * VEC - mis;
+            if (j < j_end) {
+                if (out_same_grid && tf >= 0 && tf + VEC <= L) {
+                    st_vec_nt<DT>(p.out, orow + tf, E::pack(acc));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        if (tf + e >= 0 && tf + e < L) st_elem<DT>(p.out, orow + tf + e, acc[e]);
+                }
+            }
+        }
+    }
+
+    // final_states[b, c, i] = xpad[L-(W-1)+i], bit-exact copies, by the row's first wave.
+    if (p.final_states != nullptr && seg == 0 && lane < W - 1) {
+        const int t = L - (W - 1) + lane;
+        T v = T(0.f);
+        if (t >= 0) {
+            v = ld_raw<DT>(p.x, xrow + t);
+        } else if (p.initial_states != nullptr) {
+            v = ld_raw<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
+                                                 (int64_t)c * p.init_stride_c +
+                                                 (int64_t)(t + W - 1) * p.init_stride_l);
+        }
+        st_raw<DT>(p.final_states, (int64_t)b * p.final_stride_b + (int64_t)c * p.final_stride_c +
+                                       (int64_t)lane * p.final_stride_l, v);
+    }
+}
+
+template <int DT>
+int launch_dtype(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t stream) {
+    const uint32_t blocks = (g.total_waves + (kBlock / kWave) - 1) / (kBlock / kWave);
+    switch (p.width) {
+        case 2: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        case 3: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        default: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+    }
+    return launch_status();
+}
+
+}  // namespace
+
+int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
+    const int vec = vec_elems(p.x_dtype);
+    // Worst case over row alignments: a row may start up to vec-1 elements into its grid.
+    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
+    const int64_t rows = (int64_t)p.batch * p.dim;
+    int64_t vps;
+    if (tunables().fwd_cf_vecs > 0) {
+        vps = tunables().fwd_cf_vecs;
+    } else {
+        // Enough waves to cover 256 CUs about 16 deep; otherwise one wave per row.
+        const int64_t want_segs = rows >= 4096 ? 1 : (4096 + rows - 1) / rows;
+        vps = (max_vecs + want_segs - 1) / want_segs;
+    }
+    vps = (vps + kWave - 1) / kWave * kWave;
+    if (vps < kWave) vps = kWave;
+    FwdCfGeom g;
+    g.vecs_per_seg = (int32_t)vps;
+    g.n_segs = (int32_t)((max_vecs + vps - 1) / vps);
+    const int64_t total = rows * g.n_segs;
+    if (total >= ((int64_t)1 << 25)) return CC1D_ERR_TOO_LARGE;   // total*64 threads must fit 2^31
+    g.total_waves = (uint32_t)total;
+    switch (p.x_dtype) {
+        case CC1D_F32: return launch_dtype<CC1D_F32>(p, g, stream);
+        case CC1D_F16: return launch_dtype<CC1D_F16>(p, g, stream);
+        default: return launch_dtype<CC1D_BF16>(p, g, stream);
+    }
+}
+
+}  // namespace cc1d

@@ -1,0 +1,63 @@
+// Host-side contracts between the C-ABI front (cc1d_api.cpp) and the kernel launchers
+// (one .hip file per kernel family).  A launcher is only called with parameters that
+// passed the matching cc1d_validate_*; it picks the template instance, sizes the grid
+// and returns a cc1d_status.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "cc1d.h"
+
+namespace cc1d {
+
+inline int elem_bytes(int dtype) { return dtype == CC1D_F32 ? 4 : 2; }
+inline int vec_elems(int dtype) { return 16 / elem_bytes(dtype); }
+
+// x is channel-last iff stride 1 along dim and stride > 1 along seqlen
+// (csrc/causal_conv1d.cpp:176 of the reference).
+inline bool is_channel_last(int64_t stride_c, int64_t stride_l) {
+    return stride_c == 1 && stride_l > 1;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// weight is fp32, densely packed (dim, width) and 16-byte aligned: lanes may fetch
+// their channels' taps as whole vectors.
+inline bool weights_contiguous_f32(const void *w, int w_dtype, int64_t sc, int64_t sw, int width) {
+    return w_dtype == CC1D_F32 && sw == 1 && sc == width && aligned16(w);
+}
+
+// A (batch, dim, k) states tensor can be accessed as 16-byte vectors along dim.
+inline bool states_vec_ok(const void *p, int x_dtype, int64_t sb, int64_t sc, int64_t sl) {
+    const int v = vec_elems(x_dtype);
+    return p != nullptr && sc == 1 && sb % v == 0 && sl % v == 0 && aligned16(p);
+}
+
+struct Tunables {
+    int32_t fwd_cl_rows = 0;
+    int32_t bwd_cl_rows = 0;
+    int32_t fwd_cf_vecs = 0;
+    int32_t bwd_cf_parts = 0;
+};
+Tunables &tunables();
+
+inline int launch_status() {
+    return hipGetLastError() == hipSuccess ? CC1D_OK : CC1D_ERR_LAUNCH;
+}
+
+int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream);
+int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream);
+
+size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p);
+size_t bwd_channelfirst_workspace_bytes(const cc1d_bwd_params &p);
+int launch_bwd_channellast(const cc1d_bwd_params &p, void *ws, hipStream_t stream);
+int launch_bwd_channelfirst(const cc1d_bwd_params &p, void *ws, hipStream_t stream);
+// Second stage of both backward layouts: ordered sum of the workspace planes into dweight/dbias.
+int launch_bwd_finalize(const float *ws, int n_parts, const cc1d_bwd_params &p, hipStream_t stream);
+
+int launch_update(const cc1d_update_params &p, hipStream_t stream);
+int launch_varlen_states(const cc1d_varlen_params &p, hipStream_t stream);
+
+}  // namespace cc1d

@@ -1,0 +1,96 @@
+// Varlen final-state gather for gfx950, in plain HIP.  Takes over the Triton kernel
+// _causal_conv1d_varlen_states and its launch
+// (causal_conv1d/causal_conv1d_varlen.py:8-64 of the reference).
+//
+//   states[b, :, S-k .. S) = x[end_b - k .. end_b, :],  k = min(S, end_b - start_b),
+//   states[b, :, 0 .. S-k) = 0.
+//
+// A pure copy: it moves raw bit patterns and is bit-exact.  Lanes own one 16-byte vector
+// of channels of one (sequence, state column) when x and states have unit stride along
+// dim; any other strides take the element kernel.  Rows that cu_seqlens would place
+// outside [0, total_tokens) are written as zeros instead of being read.
+#include "cc1d_device.hpp"
+#include "cc1d_internal.hpp"
+
+namespace cc1d {
+namespace {
+
+__device__ __forceinline__ int64_t cu_at(const void *cu, bool is64, int i) {
+    return is64 ? reinterpret_cast<const int64_t *>(cu)[i]
+                : (int64_t) reinterpret_cast<const int32_t *>(cu)[i];
+}
+
+// Source row of state column s of sequence b, or -1 for a zero column.
+__device__ __forceinline__ int64_t source_row(const cc1d_varlen_params &p, int b, int s) {
+    const bool is64 = p.cu_seqlens_is_int64 != 0;
+    const int64_t end = cu_at(p.cu_seqlens, is64, b + 1);
+    int64_t start = cu_at(p.cu_seqlens, is64, b);
+    if (start < end - p.state_len) start = end - p.state_len;
+    const int64_t row = end - (p.state_len - s);
+    return (row >= start && row >= 0 && row < p.total_tokens) ? row : -1;
+}
+
+template <int DT>
+__global__ void __launch_bounds__(kBlock)
+varlen_states_vec_kernel(const cc1d_varlen_params p, const uint32_t n_colgroups,
+                         const uint32_t total) {
+    constexpr int VEC = Elem<DT>::kVec;
+    const uint32_t gid = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
+    if (gid >= total) return;
+    const int c0 = (int)(gid % n_colgroups) * VEC;
+    const uint32_t bs = gid / n_colgroups;
+    const int s = (int)(bs % (uint32_t)p.state_len);
+    const int b = (int)(bs / (uint32_t)p.state_len);
+    const int64_t row = source_row(p, b, s);
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row >= 0) v = ld_vec<DT>(p.x, row * p.x_stride_t + c0);
+    st_vec<DT>(p.states, (int64_t)b * p.states_stride_b + (int64_t)s * p.states_stride_l + c0, v);
+}
+
+template <int DT>
+__global__ void __launch_bounds__(kBlock)
+varlen_states_elem_kernel(const cc1d_varlen_params p, const uint32_t total) {
+    using T = typename Elem<DT>::type;
+    const uint32_t gid = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
+    if (gid >= total) return;
+    const int c = (int)(gid % (uint32_t)p.dim);
+    const uint32_t bs = gid / (uint32_t)p.dim;
+    const int s = (int)(bs % (uint32_t)p.state_len);
+    const int b = (int)(bs / (uint32_t)p.state_len);
+    const int64_t row = source_row(p, b, s);
+    T v = T(0.f);
+    if (row >= 0) v = ld_raw<DT>(p.x, row * p.x_stride_t + (int64_t)c * p.x_stride_c);
+    st_raw<DT>(p.states, (int64_t)b * p.states_stride_b + (int64_t)c * p.states_stride_c +
+                             (int64_t)s * p.states_stride_l, v);
+}
+
+template <int DT>
+int launch_dtype(const cc1d_varlen_params &p, bool vec, hipStream_t stream) {
+    if (vec) {
+        const uint32_t ncg = (uint32_t)(p.dim / Elem<DT>::kVec);
+        const int64_t total = (int64_t)p.batch * p.state_len * ncg;
+        if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+        hipLaunchKernelGGL((varlen_states_vec_kernel<DT>), dim3((uint32_t)((total + kBlock - 1) / kBlock)),
+                           dim3(kBlock), 0, stream, p, ncg, (uint32_t)total);
+    } else {
+        const int64_t total = (int64_t)p.batch * p.state_len * p.dim;
+        if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+        hipLaunchKernelGGL((varlen_states_elem_kernel<DT>), dim3((uint32_t)((total + kBlock - 1) / kBlock)),
+                           dim3(kBlock), 0, stream, p, (uint32_t)total);
+    }
+    return launch_status();
+}
+
+}  // namespace
+
+int launch_varlen_states(const cc1d_varlen_params &p, hipStream_t stream) {
+    const int v = vec_elems(p.x_dtype);
+    const bool vec = p.dim % v == 0 && p.x_stride_c == 1 && p.x_stride_t % v == 0 && aligned16(p.x) &&
+                     p.states_stride_c == 1 && p.states_stride_b % v == 0 &&
+                     (p.state_len <= 1 || p.states_stride_l % v == 0) && aligned16(p.states);
+    // 2-byte types only differ in how bits are interpreted; the copy treats them alike.
+    return p.x_dtype == CC1D_F32 ? launch_dtype<CC1D_F32>(p, vec, stream)
+                                 : launch_dtype<CC1D_F16>(p, vec, stream);
+}
+
+}  // namespace cc1d
