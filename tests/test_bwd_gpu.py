@@ -1,0 +1,197 @@
+"""GPU parity of the backward kernels (dx, dweight, dbias, dinitial_states) against the CPU
+oracle (autograd through the PyTorch forward), through the public autograd Function and
+through the C ABI.  Grids restate tests/test_causal_conv1d.py:50-137 and :401-472 of the
+reference; determinism follows :560-575.  initial/final states are also exercised for
+channel-first, which the reference refuses.
+
+Tolerances: dx / dinitial_states as the forward (fp32 1e-5 absolute, fp16 3e-3/5e-3, bf16
+1e-2/5e-2); dweight / dbias rtol 1e-3, atol 1e-3 (long fp32 sums, summation order differs).
+"""
+import ctypes
+
+import pytest
+import torch
+
+import cabi
+from golden_io import load_case
+from helpers import (DTYPES, TOL_W, assert_close, gen, make_states, make_wb, make_x, random_seq_idx,
+                     to_dev_like)
+from oracle import causal_conv1d_oracle as orc
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+SEQLENS = [1, 2, 8, 16, 32, 64, 128, 129, 130, 151, 256, 372, 512, 784, 1024, 1134, 2048, 4096]
+
+
+def run_gpu(pkg, dev, x, w, b, dout, seq=None, init=None, dfin=None, act=None):
+    xd = to_dev_like(x, dev).requires_grad_()
+    wd = w.to(dev).requires_grad_()
+    bd = b.to(dev).requires_grad_() if b is not None else None
+    idev = init.to(dev).requires_grad_() if init is not None else None
+    res = pkg.causal_conv1d_fn(xd, wd, bd, seq_idx=None if seq is None else seq.to(dev),
+                               initial_states=idev, return_final_states=dfin is not None, activation=act)
+    if dfin is not None:
+        torch.autograd.backward(list(res), [to_dev_like(dout, dev), dfin.to(dev)])
+    else:
+        res.backward(to_dev_like(dout, dev))
+    return (xd.grad, wd.grad, None if bd is None else bd.grad, None if idev is None else idev.grad)
+
+
+def check(got, ref, dtype):
+    names = ("dx", "dweight", "dbias", "dinitial_states")
+    for name, g, r in zip(names, got, ref):
+        assert (g is None) == (r is None), name
+        if g is None:
+            continue
+        if name in ("dweight", "dbias"):
+            assert g.dtype == torch.float32
+            assert_close(g, r, what=name, tol=TOL_W)
+        else:
+            assert g.dtype == dtype
+            assert_close(g, r.to(dtype), dtype, name)
+
+
+def _grid():
+    cases, n = [], 0
+    for dim in (64, 4096 + 32):
+        for seqlen in SEQLENS:
+            for dtype in DTYPES:
+                for channel_last in (False, True):
+                    width = 2 + (n + 1) % 3
+                    has_bias = (n // 3) % 2 == 0
+                    silu = (n // 6) % 2 == 1
+                    states = (n // 12 + n) % 4            # bit 0: initial_states, bit 1: final states
+                    cases.append(pytest.param(dim, seqlen, dtype, channel_last, width, has_bias, silu, states,
+                                              id=f"d{dim}-l{seqlen}-{str(dtype)[6:]}-{'cl' if channel_last else 'cf'}"
+                                                 f"-w{width}-b{int(has_bias)}-s{int(silu)}-st{states}"))
+                    n += 1
+    return cases
+
+
+@pytest.mark.parametrize("dim,seqlen,dtype,channel_last,width,has_bias,silu,states", _grid())
+def test_bwd_matches_oracle(pkg, gpu_device, dim, seqlen, dtype, channel_last, width, has_bias, silu, states):
+    g = gen(seqlen * 5 + dim + width)
+    x = make_x(2, dim, seqlen, dtype, channel_last, g)
+    w, b = make_wb(dim, width, has_bias, g)
+    dout = make_x(2, dim, seqlen, dtype, channel_last, g, sliced=False)
+    init = make_states(2, dim, width - 1, dtype, g) if states & 1 else None
+    dfin = make_states(2, dim, width - 1, dtype, g) if states & 2 else None
+    act = "silu" if silu else None
+    ref = orc.bwd(x, w, b, dout, initial_states=init, dfinal_states=dfin, activation=act)
+    got = run_gpu(pkg, gpu_device, x, w, b, dout, init=init, dfin=dfin, act=act)
+    check(got, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim,seqlen,width,has_bias,silu", [
+    (64, 8, 2, True, True), (64, 16, 3, False, True), (64, 151, 4, True, False), (64, 372, 4, True, True),
+    (64, 1134, 3, True, True), (4128, 32, 4, True, True), (4128, 128, 2, False, False),
+    (4128, 784, 4, True, True), (4128, 2048, 3, True, True), (4128, 4096, 4, True, True),
+])
+def test_bwd_seq_idx_matches_oracle(pkg, gpu_device, dim, seqlen, width, has_bias, silu, dtype):
+    g = gen(seqlen + dim + width + 1)
+    x = make_x(3, dim, seqlen, dtype, True, g)
+    w, b = make_wb(dim, width, has_bias, g)
+    dout = make_x(3, dim, seqlen, dtype, True, g, sliced=False)
+    seq = random_seq_idx(3, seqlen, g)
+    act = "silu" if silu else None
+    ref = orc.bwd(x, w, b, dout, seq_idx=seq, activation=act)
+    got = run_gpu(pkg, gpu_device, x, w, b, dout, seq=seq, act=act)
+    check(got, ref, dtype)
+
+
+def test_bwd_seq_idx_padding_gets_no_gradient(pkg, gpu_device):
+    """The gradient of the forward as defined (exact zeros at seq_idx < 0): nothing flows
+    into or out of padding tokens.  Checked against the closed-form C restatement."""
+    g = gen(9)
+    x = make_x(3, 64, 200, torch.float32, True, g)
+    w, b = make_wb(64, 4, True, g)
+    dout = make_x(3, 64, 200, torch.float32, True, g, sliced=False)
+    seq = random_seq_idx(3, 200, g, pad=True)
+    got = run_gpu(pkg, gpu_device, x, w, b, dout, seq=seq, act="silu")
+    ref = c_oracle.bwd(x, w, b, dout, seq_idx=seq, silu=True)
+    assert torch.all(got[0].cpu()[(seq < 0).unsqueeze(1).expand(3, 64, 200)] == 0)
+    assert_close(got[0], ref[0].float(), torch.float32, "dx")
+    assert_close(got[1], ref[1].float(), what="dweight", tol=TOL_W)
+    assert_close(got[2], ref[2].float(), what="dbias", tol=TOL_W)
+
+
+def test_bwd_golden_fixture(pkg, gpu_device):
+    c = load_case("bwd")
+    for cl in (False, True):
+        lay = (lambda t: t.transpose(1, 2).contiguous().transpose(1, 2)) if cl else (lambda t: t)
+        got = run_gpu(pkg, gpu_device, lay(c["x"]), c["weight"], c["bias"], lay(c["dout"]),
+                      init=c["initial_states"], dfin=c["dfinal_states"], act="silu")
+        check(got, (c["dx"], c["dweight"], c["dbias"], c["dinitial_states"]), torch.float32)
+
+
+@pytest.mark.parametrize("channel_last", [False, True])
+def test_bwd_is_bit_reproducible(pkg, gpu_device, channel_last):
+    """Five runs, identical bits in dx, dweight and dbias (the reduction is a fixed-order
+    two-stage sum; tests/test_causal_conv1d.py:560-575 asks this of deterministic mode)."""
+    g = gen(1234)
+    x = make_x(4, 1024, 2048, torch.bfloat16, channel_last, g, sliced=False)
+    w, b = make_wb(1024, 4, True, g)
+    dout = make_x(4, 1024, 2048, torch.bfloat16, channel_last, g, sliced=False)
+    first = run_gpu(pkg, gpu_device, x, w, b, dout, act="silu")
+    for _ in range(4):
+        again = run_gpu(pkg, gpu_device, x, w, b, dout, act="silu")
+        for a, f in zip(again[:3], first[:3]):
+            assert torch.equal(a, f)
+    ref = orc.bwd(x, w, b, dout, activation="silu")
+    check(first, ref, torch.bfloat16)
+
+
+@pytest.mark.parametrize("channel_last", [False, True])
+def test_bwd_c_abi_accumulates_into_dweight(gpu_device, cc1d_lib, channel_last):
+    """Through the C ABI with a caller-owned workspace: dweight / dbias are added to, as the
+    reference's atomicAdd / add_ do (csrc/causal_conv1d_bwd.cu:243; causal_conv1d.cpp:452)."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    g = gen(77)
+    x = make_x(2, 64, 500, torch.float32, channel_last, g, sliced=False)
+    dout = make_x(2, 64, 500, torch.float32, channel_last, g, sliced=False)
+    w, b = make_wb(64, 3, True, g)
+    ref = orc.bwd(x, w, b, dout, activation="silu")
+    xd, dd, wd, bd = (t.to(dev) for t in (x, dout, w, b))
+    dx = torch.empty_like(xd)
+    dw = torch.full((64, 3), 2.0, device=dev)
+    db = torch.full((64,), -1.0, device=dev)
+    p = cabi.bwd_params(xd, wd, bd, dd, dx, dw, db, True)
+    need = ctypes.c_size_t()
+    assert lib.cc1d_bwd_workspace_bytes(ctypes.byref(p), ctypes.byref(need)) == 0
+    ws = torch.empty(max(16, need.value), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    if need.value:
+        assert lib.cc1d_bwd(ctypes.byref(p), ws.data_ptr(), need.value - 1, stream) == -13
+    st = lib.cc1d_bwd(ctypes.byref(p), ws.data_ptr(), need.value, stream)
+    assert st == 0, lib.cc1d_strerror(st)
+    torch.cuda.synchronize()
+    assert_close(dx, ref[0], torch.float32, "dx")
+    assert_close(dw - 2.0, ref[1], what="dweight", tol=TOL_W)
+    assert_close(db + 1.0, ref[2], what="dbias", tol=TOL_W)
+
+
+def test_bwd_full_size_fp16_channel_first_with_states(pkg, gpu_device):
+    """The backward configuration at full size: fp16 (4, 4096, 8192) channel-first, width 4,
+    SiLU, initial_states and a gradient on final_states.  Channels are independent, so a
+    handful of channels is checked exactly against the oracle at full batch and length;
+    the whole dx is checked through linearity in dout."""
+    import bench
+    cfg = bench.config_c4()
+    dev = gpu_device
+    got = run_gpu(pkg, dev, cfg["x"], cfg["weight"], cfg["bias"], cfg["dout"],
+                  init=cfg["initial_states"], dfin=cfg["dfinal_states"], act="silu")
+    ch = torch.tensor([0, 1, 63, 64, 2047, 4095])
+    ref = orc.bwd(cfg["x"][:, ch], cfg["weight"][ch], cfg["bias"][ch], cfg["dout"][:, ch],
+                  initial_states=cfg["initial_states"][:, ch], dfinal_states=cfg["dfinal_states"][:, ch],
+                  activation="silu")
+    chd = ch.to(dev)
+    sub = (got[0][:, chd], got[1][chd], got[2][chd], got[3][:, chd])
+    check(sub, ref, torch.float16)
+    # linearity: gradients for (2*dout, 2*dfinal) are exactly twice those for (dout, dfinal)
+    got2 = run_gpu(pkg, dev, cfg["x"], cfg["weight"], cfg["bias"], cfg["dout"] * 2,
+                   init=cfg["initial_states"], dfin=cfg["dfinal_states"] * 2, act="silu")
+    assert_close(got2[0], got[0].float() * 2, torch.float16, "dx linearity")
+    assert_close(got2[1], got[1] * 2, what="dweight linearity", tol=TOL_W)

@@ -1,0 +1,202 @@
+"""GPU parity of the forward kernels against the CPU oracle, through the public Python API
+(package -> torch extension -> C ABI -> HIP kernels) and, for one case, through the C ABI
+directly.  The grids restate tests/test_causal_conv1d.py:50-137 (dense), :401-472 (seq_idx)
+and :474-557 (seq_idx with padding) of the reference; initial/final states are also
+exercised for channel-first, which the reference refuses.
+
+Tolerances: fp32 |diff| <= 1e-5; fp16 rtol 3e-3 / atol 5e-3; bf16 rtol 1e-2 / atol 5e-2;
+final_states, a pure copy, bit-exact.
+"""
+import ctypes
+
+import pytest
+import torch
+
+import cabi
+from golden_io import load_case
+from helpers import (DTYPES, TOL, assert_close, gen, make_states, make_wb, make_x, random_seq_idx,
+                     to_dev_like)
+from oracle import causal_conv1d_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+SEQLENS = [1, 2, 8, 16, 32, 64, 128, 129, 130, 151, 256, 372, 512, 784, 1024, 1134, 2048, 4096]
+
+
+def _grid():
+    """Every (dim, seqlen, dtype, layout); width / bias / SiLU / states rotate through all
+    their combinations across the grid."""
+    cases, n = [], 0
+    for dim in (64, 4096 + 32):
+        for seqlen in SEQLENS:
+            for dtype in DTYPES:
+                for channel_last in (False, True):
+                    width = 2 + n % 3
+                    has_bias = (n // 3) % 2 == 0
+                    silu = (n // 6) % 2 == 0
+                    states = (n // 12 + n) % 4            # 0 none, 1 initial, 2 final, 3 both
+                    cases.append(pytest.param(dim, seqlen, dtype, channel_last, width, has_bias, silu, states,
+                                              id=f"d{dim}-l{seqlen}-{str(dtype)[6:]}-{'cl' if channel_last else 'cf'}"
+                                                 f"-w{width}-b{int(has_bias)}-s{int(silu)}-st{states}"))
+                    n += 1
+    return cases
+
+
+@pytest.mark.parametrize("dim,seqlen,dtype,channel_last,width,has_bias,silu,states", _grid())
+def test_fwd_matches_oracle(pkg, gpu_device, dim, seqlen, dtype, channel_last, width, has_bias, silu, states):
+    g = gen(seqlen * 7 + dim + width)
+    x = make_x(2, dim, seqlen, dtype, channel_last, g)
+    w, b = make_wb(dim, width, has_bias, g)
+    init = make_states(2, dim, width - 1, dtype, g) if states & 1 else None
+    want_final = bool(states & 2)
+    act = "silu" if silu else None
+
+    ref = orc.fwd(x, w, b, initial_states=init, return_final_states=want_final, activation=act)
+    got = pkg.causal_conv1d_fn(to_dev_like(x, gpu_device), w.to(gpu_device),
+                               None if b is None else b.to(gpu_device),
+                               initial_states=None if init is None else init.to(gpu_device),
+                               return_final_states=want_final, activation=act)
+    if want_final:
+        (got, got_fin), (ref, ref_fin) = got, ref
+        assert got_fin.shape == ref_fin.shape and got_fin.stride(1) == 1
+        assert torch.equal(got_fin.cpu(), ref_fin), "final_states must be an exact copy"
+    assert got.dtype == dtype and got.shape == x.shape
+    assert_close(got, ref, dtype, "out")
+
+
+@pytest.mark.parametrize("pad", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim,seqlen,width,has_bias,silu", [
+    (64, 8, 2, True, True), (64, 16, 3, False, True), (64, 151, 4, True, False), (64, 372, 4, True, True),
+    (64, 1134, 3, True, True), (4128, 32, 4, True, True), (4128, 128, 2, False, False),
+    (4128, 784, 4, True, True), (4128, 2048, 3, True, True), (4128, 4096, 4, True, True),
+])
+def test_fwd_seq_idx_matches_per_segment_oracle(pkg, gpu_device, dim, seqlen, width, has_bias, silu, dtype, pad):
+    g = gen(seqlen + dim + width)
+    x = make_x(3, dim, seqlen, dtype, True, g)
+    w, b = make_wb(dim, width, has_bias, g)
+    seq = random_seq_idx(3, seqlen, g, pad=pad)
+    act = "silu" if silu else None
+    ref = orc.fwd_seq_idx(x, w, b, seq, activation=act)
+    got = pkg.causal_conv1d_fn(to_dev_like(x, gpu_device), w.to(gpu_device),
+                               None if b is None else b.to(gpu_device),
+                               seq_idx=seq.to(gpu_device), activation=act)
+    assert_close(got, ref, dtype, "out")
+    if pad:
+        assert torch.all(got.cpu()[(seq < 0).unsqueeze(1).expand_as(got)] == 0), "padding must be exact zeros"
+
+
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("channel_last", [False, True])
+def test_fwd_all_nine_dtype_pairs(pkg, gpu_device, dtype, w_dtype, channel_last):
+    """x dtype x weight dtype (csrc/causal_conv1d_fwd.cu:383-401); the oracle computes in the
+    weight dtype, the kernel in fp32, so 16-bit weights get the 16-bit tolerance."""
+    g = gen(3)
+    x = make_x(2, 72, 200, dtype, channel_last, g, sliced=False)
+    w, b = make_wb(72, 4, True, g, w_dtype)
+    ref = orc.fwd(x.float(), w.float(), b.float(), activation="silu").to(dtype)
+    got = pkg.causal_conv1d_fn(x.to(gpu_device), w.to(gpu_device), b.to(gpu_device), activation="silu")
+    assert_close(got, ref, dtype, "out")
+    # non-contiguous weight (a transposed view) takes the strided tap loads
+    wt = w.t().contiguous().t()
+    got2 = pkg.causal_conv1d_fn(x.to(gpu_device), wt.to(gpu_device).t().contiguous().t(), b.to(gpu_device), activation="silu")
+    assert torch.equal(got.cpu(), got2.cpu())
+
+
+def test_fwd_golden_fixtures(pkg, gpu_device):
+    d = gpu_device
+    c = load_case("fwd_c1")
+    got = pkg.causal_conv1d_fn(c["x"].to(d), c["weight"].to(d), c["bias"].to(d), activation="silu")
+    assert_close(got, c["out"], torch.float32, "fwd_c1")
+    c = load_case("fwd_states")
+    for cl in (False, True):
+        x = c["x"].transpose(1, 2).contiguous().transpose(1, 2) if cl else c["x"]
+        got, fin = pkg.causal_conv1d_fn(x.to(d), c["weight"].to(d), c["bias"].to(d),
+                                        initial_states=c["initial_states"].to(d), return_final_states=True)
+        assert_close(got, c["out"], torch.bfloat16, "fwd_states")
+        assert torch.equal(fin.cpu(), c["final_states"])
+    c = load_case("fwd_seq")
+    x = c["x"].transpose(1, 2).contiguous().transpose(1, 2)
+    got = pkg.causal_conv1d_fn(x.to(d), c["weight"].to(d), c["bias"].to(d), seq_idx=c["seq_idx"].to(d), activation="silu")
+    assert_close(got, c["out"], torch.float16, "fwd_seq")
+
+
+def test_fwd_chunking_is_bit_exact_at_prefill_size(pkg, gpu_device):
+    """Size-independent property at the full Mamba-2 2.7B prefill shape: running the
+    sequence in two chunks, handing final_states over as initial_states, reproduces the
+    unchunked output bit for bit; and a slice of rows agrees with the oracle."""
+    import bench
+    cfg = bench.config_c2()
+    d = gpu_device
+    x, w, b = cfg["x"].to(d), cfg["weight"].to(d), cfg["bias"].to(d)
+    whole = pkg.causal_conv1d_fn(x, w, b, activation="silu")
+    cut = 1000                                             # rows keep their 8-element alignment
+    head, fin = pkg.causal_conv1d_fn(x[:, :, :cut], w, b, return_final_states=True, activation="silu")
+    tail = pkg.causal_conv1d_fn(x[:, :, cut:], w, b, initial_states=fin, activation="silu")
+    assert torch.equal(torch.cat([head, tail], dim=2), whole)
+    ref = orc.fwd(cfg["x"][3:4], cfg["weight"], cfg["bias"], activation="silu")
+    assert_close(whole[3:4], ref, torch.bfloat16, "row 3")
+    seq = cfg["seq_idx"].to(d)
+    got = pkg.causal_conv1d_fn(x, w, b, seq_idx=seq, activation="silu")
+    ref = orc.fwd_seq_idx(cfg["x"][5:6], cfg["weight"], cfg["bias"], cfg["seq_idx"][5:6], activation="silu")
+    assert_close(got[5:6], ref, torch.bfloat16, "row 5 with seq_idx")
+    # a single sub-sequence id per row is the dense result
+    assert torch.equal(pkg.causal_conv1d_fn(x, w, b, seq_idx=torch.zeros_like(seq), activation="silu"), whole)
+
+
+def test_fwd_rows_per_run_does_not_change_results(pkg, gpu_device, cc1d_lib):
+    """Every run length of the channel-last walk gives the same bits."""
+    lib = cabi.declare(cc1d_lib)
+    g = gen(11)
+    x = make_x(2, 264, 333, torch.bfloat16, True, g).to(gpu_device)
+    w, b = (t.to(gpu_device) for t in make_wb(264, 4, True, g))
+    seq = random_seq_idx(2, 333, g).to(gpu_device)
+    outs = []
+    try:
+        for rows in (4, 8, 32, 64, 128, 1024):
+            assert lib.cc1d_set_tunable(b"fwd_cl_rows", rows) == 0
+            outs.append(pkg.causal_conv1d_fn(x, w, b, seq_idx=seq, activation="silu").cpu())
+    finally:
+        lib.cc1d_set_tunable(b"fwd_cl_rows", 0)
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
+def test_fwd_through_the_c_abi_on_a_side_stream(gpu_device, cc1d_lib):
+    """The C ABI alone: raw pointers, element strides and an explicit stream handle."""
+    lib = cabi.declare(cc1d_lib)
+    g = gen(5)
+    x = make_x(2, 64, 300, torch.float32, False, g, sliced=False)
+    w, b = make_wb(64, 4, True, g)
+    init = make_states(2, 64, 3, torch.float32, g)
+    ref, ref_fin = orc.fwd(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+    xd, wd, bd, idev = (t.to(gpu_device) for t in (x, w, b, init))
+    out, fin = torch.empty_like(xd), torch.empty(2, 64, 3, device=gpu_device)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    p = cabi.fwd_params(xd, wd, bd, out, True, initial_states=idev, final_states=fin)
+    st = lib.cc1d_fwd(ctypes.byref(p), ctypes.c_void_p(stream.cuda_stream))
+    assert st == 0, lib.cc1d_strerror(st)
+    stream.synchronize()
+    assert_close(out, ref, torch.float32, "out")
+    assert torch.equal(fin.cpu(), ref_fin)
+
+
+def test_fwd_error_behaviour(pkg, gpu_device):
+    d = gpu_device
+    x = torch.zeros(2, 16, 32, device=d)
+    with pytest.raises(RuntimeError, match="width between 2 and 4"):
+        pkg.causal_conv1d_fn(x, torch.zeros(16, 5, device=d))
+    with pytest.raises(NotImplementedError):
+        pkg.causal_conv1d_fn(x, torch.zeros(16, 4, device=d), activation="relu")
+    xcl = torch.zeros(2, 32, 12, device=d).transpose(1, 2)
+    with pytest.raises(RuntimeError, match="divisible by 8"):
+        pkg.causal_conv1d_fn(xcl, torch.zeros(12, 4, device=d))
+    with pytest.raises(RuntimeError, match="channel last"):
+        pkg.causal_conv1d_fn(x, torch.zeros(16, 4, device=d), seq_idx=torch.zeros(2, 32, dtype=torch.int32, device=d))
+    with pytest.raises(AssertionError):
+        pkg.causal_conv1d_fn(xcl, torch.zeros(12, 4, device=d), seq_idx=torch.zeros(2, 32, dtype=torch.int32, device=d),
+                             return_final_states=True)
+    empty = pkg.causal_conv1d_fn(torch.zeros(0, 16, 32, device=d), torch.zeros(16, 4, device=d))
+    assert empty.shape == (0, 16, 32)

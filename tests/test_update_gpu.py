@@ -1,0 +1,144 @@
+"""GPU parity of the decode-step update against the CPU oracle.  Grids restate
+tests/test_causal_conv1d.py:140-183 (plain), :185-233 (conv_state_indices) and :236-321
+(negative indices = padding) of the reference.  conv_state must be bit-exact; out within
+the forward tolerances."""
+import ctypes
+
+import pytest
+import torch
+
+import cabi
+from golden_io import load_case
+from helpers import DTYPES, assert_close, gen, make_wb
+from oracle import causal_conv1d_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _grid():
+    cases, n = [], 0
+    for dim in (2048, 2048 + 16, 4096):
+        for width in (2, 3, 4):
+            for seqlen in (1, 4, 5):
+                for circular in (False, True):
+                    for dtype in DTYPES:
+                        has_bias = n % 2 == 0
+                        silu = (n // 2) % 2 == 0
+                        cases.append(pytest.param(dim, width, seqlen, circular, dtype, has_bias, silu,
+                                                  id=f"d{dim}-w{width}-l{seqlen}-c{int(circular)}-{str(dtype)[6:]}"
+                                                     f"-b{int(has_bias)}-s{int(silu)}"))
+                        n += 1
+    return cases
+
+
+def _inputs(dim, width, seqlen, dtype, has_bias, g, batch=64, entries=None, state_dim_last=True):
+    x = torch.randn(batch, seqlen, dim, generator=g).to(dtype).transpose(-1, -2)
+    state_len = int(torch.randint(width - 1, width + 10, (1,), generator=g))
+    n = entries or batch
+    if state_dim_last:
+        st = torch.randn(n, state_len, dim, generator=g).to(dtype).transpose(-1, -2)
+    else:
+        st = torch.randn(n, dim, state_len, generator=g).to(dtype)
+    w, b = make_wb(dim, width, has_bias, g)
+    return x, st, w, b
+
+
+@pytest.mark.parametrize("dim,width,seqlen,circular,dtype,has_bias,silu", _grid())
+def test_update_matches_oracle(pkg, gpu_device, dim, width, seqlen, circular, dtype, has_bias, silu):
+    g = gen(dim + width * 10 + seqlen)
+    x, st, w, b = _inputs(dim, width, seqlen, dtype, has_bias, g)
+    cs = torch.randint(0, 1024, (64,), generator=g, dtype=torch.int32) if circular else None
+    act = "silu" if silu else None
+    st_ref = st.clone()
+    ref = orc.update(x, st_ref, w, b, activation=act, cache_seqlens=cs)
+    d = gpu_device
+    st_dev = st.to(d)
+    got = pkg.causal_conv1d_update(x.to(d), st_dev, w.to(d), None if b is None else b.to(d), activation=act,
+                                   cache_seqlens=None if cs is None else cs.to(d))
+    assert torch.equal(st_dev.cpu(), st_ref), "conv_state must be bit-exact"
+    assert_close(got, ref, dtype, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("circular", [False, True])
+@pytest.mark.parametrize("dim,width,seqlen", [(2048, 4, 1), (2064, 3, 4), (4096, 2, 5), (2048, 4, 5)])
+def test_update_with_batch_gather_and_padding(pkg, gpu_device, dim, width, seqlen, circular, dtype):
+    g = gen(dim + width + seqlen + 1)
+    x, st, w, b = _inputs(dim, width, seqlen, dtype, True, g, entries=640)
+    idx = torch.randperm(640, generator=g)[:64].to(torch.int32)
+    idx[torch.randperm(64, generator=g)[:32]] = -1                   # half the requests are padding
+    cs = torch.randint(0, 1024, (64,), generator=g, dtype=torch.int32) if circular else None
+    st_ref = st.clone()
+    ref = orc.update(x, st_ref, w, b, activation="silu", cache_seqlens=cs, conv_state_indices=idx)
+    d = gpu_device
+    st_dev = st.to(d)
+    got = pkg.causal_conv1d_update(x.to(d), st_dev, w.to(d), b.to(d), activation="silu",
+                                   cache_seqlens=None if cs is None else cs.to(d), conv_state_indices=idx.to(d))
+    assert torch.equal(st_dev.cpu(), st_ref), "gathered rows exact, every other row untouched"
+    assert torch.all(got.cpu()[idx < 0] == 0), "padding requests must output exact zeros"
+    assert_close(got, ref, dtype, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("circular", [False, True])
+def test_update_other_layouts_take_the_element_kernel(pkg, gpu_device, dtype, circular):
+    """State stored (batch, dim, state_len)-contiguous, x (batch, dim) 2-D, odd dim."""
+    g = gen(31)
+    dim, width = 2052, 4
+    x = torch.randn(16, dim, generator=g).to(dtype)
+    st = torch.randn(16, dim, 7, generator=g).to(dtype)
+    w, b = make_wb(dim, width, True, g)
+    cs = torch.randint(0, 1024, (16,), generator=g, dtype=torch.int32) if circular else None
+    st_ref = st.clone()
+    ref = orc.update(x, st_ref, w, b, activation="silu", cache_seqlens=cs)
+    d = gpu_device
+    st_dev = st.to(d)
+    got = pkg.causal_conv1d_update(x.to(d), st_dev, w.to(d), b.to(d), activation="silu",
+                                   cache_seqlens=None if cs is None else cs.to(d))
+    assert got.shape == (16, dim)
+    assert torch.equal(st_dev.cpu(), st_ref)
+    assert_close(got, ref, dtype, "out")
+
+
+def test_update_golden_and_decode_loop(pkg, gpu_device):
+    d = gpu_device
+    for case in ("update_linear", "update_circular"):
+        c = load_case(case)
+        lay = lambda t: t.transpose(1, 2).contiguous().transpose(1, 2)
+        st = lay(c["conv_state"]).to(d)
+        cs = c.get("cache_seqlens")
+        got = pkg.causal_conv1d_update(lay(c["x"]).to(d), st, c["weight"].to(d), c["bias"].to(d), activation="silu",
+                                       cache_seqlens=None if cs is None else cs.to(d))
+        assert torch.equal(st.cpu(), c["conv_state_after"])
+        assert_close(got, c["out"], torch.bfloat16, case)
+    # token-by-token decoding reproduces the prefill forward (fp32, so nearly exact)
+    g = gen(8)
+    x = torch.randn(3, 40, 128, generator=g).transpose(1, 2)
+    w, b = make_wb(128, 4, True, g)
+    whole = pkg.causal_conv1d_fn(x.to(d), w.to(d), b.to(d), activation="silu")
+    state = torch.zeros(3, 3, 128, device=d).transpose(1, 2)
+    steps = [pkg.causal_conv1d_update(x[:, :, t].to(d), state, w.to(d), b.to(d), activation="silu") for t in range(40)]
+    assert_close(torch.stack(steps, dim=-1), whole.cpu(), torch.float32, "decode loop")
+    assert torch.equal(state.cpu(), x[:, :, -3:])
+
+
+@pytest.mark.parametrize("circular", [False, True])
+def test_update_full_decode_shape_through_the_c_abi(gpu_device, cc1d_lib, circular):
+    """bf16 (256, 5376, 1) with state (256, 5376, 3) linear / (256, 5376, 8) circular, called
+    through the C ABI; the whole result is compared with the oracle."""
+    import bench
+    lib = cabi.declare(cc1d_lib)
+    cfg = bench.config_c3(circular)
+    st_ref = cfg["conv_state"].clone()
+    ref = orc.update(cfg["x"], st_ref, cfg["weight"], cfg["bias"], activation="silu",
+                     cache_seqlens=cfg.get("cache_seqlens"))
+    d = gpu_device
+    x, st, w, b = (cfg[k].to(d) for k in ("x", "conv_state", "weight", "bias"))
+    cs = cfg["cache_seqlens"].to(d) if circular else None
+    out = torch.empty_like(x)
+    p = cabi.update_params(x, st, w, b, out, True, cache_seqlens=cs)
+    rc = lib.cc1d_update(ctypes.byref(p), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.cc1d_strerror(rc)
+    torch.cuda.synchronize()
+    assert torch.equal(st.cpu(), st_ref)
+    assert_close(out, ref, torch.bfloat16, "out")
