@@ -299,6 +299,8 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--rows", type=int, default=0, help="override rows per lane run (sweeps)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain device copy of x (a kernel of known size, to scale profiler counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
@@ -324,6 +326,13 @@ def main():
         ext.causal_conv1d_fwd(x, w, b, seq, None, out, None, True)
 
     us, wall_us = time_gpu(step, args.steps, args.warmup)
+    if args.copy_probe:
+        flat_src = torch.empty(x.numel(), dtype=x.dtype, device=dev).normal_()
+        flat_dst = torch.empty_like(flat_src)
+        copy_us, _ = time_gpu(lambda i: flat_dst.copy_(flat_src), args.steps, args.warmup)
+        print("copy probe: %d bytes read + %d bytes written per launch, %.2f us" %
+              (nbytes(flat_src), nbytes(flat_dst), copy_us), file=sys.stderr)
+        del flat_src, flat_dst
 
     # Parity of what was just timed, against the oracle on a slice small enough to be quick.
     from oracle import causal_conv1d_oracle as orc

@@ -51,7 +51,8 @@ HIP_FLAGS = [
 
 def _run(cmd):
     print("+", " ".join(shlex.quote(c) for c in cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # A compile that does not finish in ten minutes is stuck in the compiler, not slow.
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
     out = "\n".join(l for l in res.stdout.splitlines()
                     if "packed-fp32-ops" not in l and l.strip())
     if out:

@@ -58,7 +58,10 @@ template <> struct Elem<CC1D_F16> {
     static constexpr int kBytes = 2;
     static constexpr bool kPreciseAct = false;
     static __device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
-    static __device__ __forceinline__ _Float16 from_float(float v) { return (_Float16)v; }
+    static __device__ __forceinline__ _Float16 from_float(float v) {
+        asm("" : "+v"(v));                  // no fused round-to-fp16 multiply (see Pack::pack)
+        return (_Float16)v;
+    }
     static __device__ __forceinline__ void unpack(const u32x4 &r, float (&f)[8]) {
         const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
@@ -72,9 +75,11 @@ template <> struct Elem<CC1D_F16> {
         uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            float lo = f[2 * i], hi = f[2 * i + 1];
+            asm("" : "+v"(lo), "+v"(hi));     // no fused round-to-fp16 multiply (see Pack::pack)
             f16x2 h;
-            h.x = (_Float16)f[2 * i];
-            h.y = (_Float16)f[2 * i + 1];
+            h.x = (_Float16)lo;
+            h.y = (_Float16)hi;
             w[i] = bitcast<uint32_t>(h);
         }
         u32x4 r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
@@ -107,6 +112,76 @@ template <> struct Elem<CC1D_BF16> {
             w[i] = bitcast<uint32_t>(h);
         }
         u32x4 r; r.x = w[0]; r.y = w[1]; r.z = w[2]; r.w = w[3];
+        return r;
+    }
+};
+
+// ---------------------------------------------------------------------------------
+// CH channels of one row held by one lane: a 16-byte or an 8-byte register vector.
+// ---------------------------------------------------------------------------------
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <int BYTES> struct RawBytes;
+template <> struct RawBytes<16> { using type = u32x4; };
+template <> struct RawBytes<8> { using type = u32x2; };
+
+template <int DT, int CH>
+struct Pack {
+    static constexpr int kBytes = CH * Elem<DT>::kBytes;
+    static constexpr int kDwords = kBytes / 4;
+    using raw_t = typename RawBytes<kBytes>::type;
+
+    static __device__ __forceinline__ raw_t zero() {
+        raw_t r;
+#pragma unroll
+        for (int i = 0; i < kDwords; ++i) r[i] = 0u;
+        return r;
+    }
+    static __device__ __forceinline__ void unpack(const raw_t &r, float (&f)[CH]) {
+        if constexpr (DT == CC1D_F32) {
+#pragma unroll
+            for (int i = 0; i < kDwords; ++i) f[i] = bitcast<float>(r[i]);
+        } else if constexpr (DT == CC1D_BF16) {
+#pragma unroll
+            for (int i = 0; i < kDwords; ++i) {
+                f[2 * i] = bitcast<float>(r[i] << 16);
+                f[2 * i + 1] = bitcast<float>(r[i] & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kDwords; ++i) {
+                const f16x2 h = bitcast<f16x2>(r[i]);
+                f[2 * i] = (float)h.x;
+                f[2 * i + 1] = (float)h.y;
+            }
+        }
+    }
+    static __device__ __forceinline__ raw_t pack(const float (&f)[CH]) {
+        raw_t r;
+        if constexpr (DT == CC1D_F32) {
+#pragma unroll
+            for (int i = 0; i < kDwords; ++i) r[i] = bitcast<uint32_t>(f[i]);
+        } else if constexpr (DT == CC1D_BF16) {
+#pragma unroll
+            for (int i = 0; i < kDwords; ++i) {
+                bf16x2 h;                   // round-to-nearest-even: v_cvt_pk_bf16_f32
+                h.x = (__bf16)f[2 * i];
+                h.y = (__bf16)f[2 * i + 1];
+                r[i] = bitcast<uint32_t>(h);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kDwords; ++i) {
+                // The empty asm keeps the compiler from folding the producing multiply
+                // into a mixed-precision fma that rounds to fp16 in one step: with it every
+                // code path rounds fp32 -> fp16 the same way and gives the same bits.
+                float lo = f[2 * i], hi = f[2 * i + 1];
+                asm("" : "+v"(lo), "+v"(hi));
+                f16x2 h;
+                h.x = (_Float16)lo;
+                h.y = (_Float16)hi;
+                r[i] = bitcast<uint32_t>(h);
+            }
+        }
         return r;
     }
 };
@@ -174,17 +249,15 @@ __device__ __forceinline__ void load_weights(const void *weight, const void *bia
                                              int64_t stride_c, int64_t stride_w,
                                              bool contiguous_f32, int c0,
                                              float (&wv)[NCH][W], float (&bv)[NCH]) {
-    static_assert((NCH * W) % 4 == 0, "NCH*W floats must be whole 16-byte vectors");
     if (contiguous_f32) {
+        // NCH*W consecutive floats starting at a multiple of NCH floats: the compiler
+        // merges them into the widest loads the alignment allows.
+        constexpr int kAlign = NCH * 4 > 16 ? 16 : NCH * 4;
+        const float *src = static_cast<const float *>(__builtin_assume_aligned(
+            reinterpret_cast<const float *>(weight) + (int64_t)c0 * W, kAlign));
         float flat[NCH * W];
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(
-            reinterpret_cast<const float *>(weight) + (int64_t)c0 * W);
 #pragma unroll
-        for (int i = 0; i < NCH * W / 4; ++i) {
-            u32x4 r = src[i];
-            flat[4 * i] = bitcast<float>(r.x); flat[4 * i + 1] = bitcast<float>(r.y);
-            flat[4 * i + 2] = bitcast<float>(r.z); flat[4 * i + 3] = bitcast<float>(r.w);
-        }
+        for (int i = 0; i < NCH * W; ++i) flat[i] = src[i];
 #pragma unroll
         for (int j = 0; j < NCH; ++j)
 #pragma unroll

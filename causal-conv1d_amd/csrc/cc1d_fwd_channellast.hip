@@ -3,195 +3,301 @@
 // (csrc/causal_conv1d_fwd.cu:205-381 of the reference).
 //
 // Design.  The stencil runs along seqlen, which is the strided axis, so nothing has to
-// be transposed: a lane owns one 16-byte vector of channels (8 x 16-bit or 4 x fp32),
-// keeps that vector's W taps and bias in registers and walks down a run of consecutive
-// rows with a (W-1)-row sliding window held in registers as fp32.  Per row that is one
-// 16-byte load and one 16-byte store per lane, both fully coalesced along dim, no LDS
-// and no barrier.  The only re-read is the (W-1)-row halo in front of each run.
+// be transposed: a lane owns CH adjacent channels (one 8- or 16-byte vector), keeps their
+// W taps and bias in registers and walks down a run of consecutive rows with a
+// (W-1)-row sliding window held in registers as fp32.  Per row that is one vector load
+// and one vector store per lane, both fully coalesced along dim, no LDS and no barrier.
+// The only re-read is the (W-1)-row halo in front of each run.
 //
-// Work items (batch, run, vector-column) are laid out flat over the grid, so every lane
-// is busy for any dim that is a multiple of the vector width; lanes of one wave may sit
-// in different runs, which is why seq_idx is tracked per lane.
+// Work items (batch, run, vector-column) are laid out flat, so every lane is busy for
+// any dim that is a multiple of CH; lanes of one wave may sit in different runs, which is
+// why seq_idx is tracked per lane.  Workgroups are renumbered so that each of the 8 XCDs
+// (hardware hands workgroups to XCDs round-robin) walks a contiguous slice of that flat
+// order: the run that follows another along seqlen then executes on the same XCD, close
+// in time, and its halo rows are found in that XCD's L2 instead of being fetched from
+// HBM twice.  For the same reason the halo rows and the last rows of a run are accessed
+// with the normal cache policy while everything else streams through (non-temporal).
+#include <type_traits>
+
 #include "cc1d_device.hpp"
 #include "cc1d_internal.hpp"
 
+// Rows per register set; two sets are in flight per lane.
 #ifndef CC1D_FWD_CL_UNROLL
-#define CC1D_FWD_CL_UNROLL 4      // rows in flight per lane (and prefetched one group ahead)
+#define CC1D_FWD_CL_UNROLL 4
 #endif
-#ifndef CC1D_FWD_CL_NT
-#define CC1D_FWD_CL_NT 1          // streaming (non-temporal) row loads and stores
+// Workgroups per CU the register budget must allow, for 16- and 8-byte lanes.
+#ifndef CC1D_FWD_CL_OCC16
+#define CC1D_FWD_CL_OCC16 2
+#endif
+#ifndef CC1D_FWD_CL_OCC8
+#define CC1D_FWD_CL_OCC8 4
 #endif
 
 namespace cc1d {
 namespace {
 
+constexpr int kXcds = 8;
+
 struct FwdClGeom {
-    int32_t rows_per_run;     // T, a multiple of the unroll factor
+    int32_t rows_per_run;     // T, a multiple of twice the unroll factor
     int32_t n_runs;           // ceil(seqlen / T)
-    int32_t n_colgroups;      // dim / kVec
+    int32_t n_colgroups;      // dim / CH
     uint32_t total;           // batch * n_runs * n_colgroups work items
+    uint32_t blocks_per_xcd;  // grid size / 8
     int32_t w_fast;           // weights_contiguous_f32
-    int32_t init_vec;         // states_vec_ok(initial_states)
-    int32_t final_vec;        // states_vec_ok(final_states)
+    int32_t seq_vec;          // seq_idx rows may be read as 16-byte vectors
 };
 
-template <int DT>
-struct alignas(16) RawVec {
-    typename Elem<DT>::type v[Elem<DT>::kVec];
+template <int DT, int CH>
+struct alignas(CH * Elem<DT>::kBytes) RawElems {
+    typename Elem<DT>::type v[CH];
 };
 
-// One (batch, l) row of a (batch, dim, k) states tensor, channels c0 .. c0+kVec.
-template <int DT>
-__device__ __forceinline__ u32x4 load_state_row(const void *base, int64_t sb, int64_t sc,
-                                                int64_t sl, int b, int c0, int l, bool vec) {
-    if (vec) return ld_vec<DT>(base, (int64_t)b * sb + (int64_t)l * sl + c0);
-    RawVec<DT> r;
+// CH channels of one (batch, l) row of a (batch, dim, k) states tensor.
+template <int DT, int CH>
+__device__ __forceinline__ typename Pack<DT, CH>::raw_t
+load_state_row(const void *base, int64_t sb, int64_t sc, int64_t sl, int b, int c0, int l) {
+    using T = typename Elem<DT>::type;
+    using raw_t = typename Pack<DT, CH>::raw_t;
+    const T *row = reinterpret_cast<const T *>(base) + (int64_t)b * sb + (int64_t)l * sl;
+    if (sc == 1 && (reinterpret_cast<uintptr_t>(row + c0) % sizeof(raw_t)) == 0)
+        return *reinterpret_cast<const raw_t *>(row + c0);
+    RawElems<DT, CH> r;
 #pragma unroll
-    for (int j = 0; j < Elem<DT>::kVec; ++j)
-        r.v[j] = ld_raw<DT>(base, (int64_t)b * sb + (int64_t)(c0 + j) * sc + (int64_t)l * sl);
-    return bitcast<u32x4>(r);
+    for (int j = 0; j < CH; ++j) r.v[j] = row[(int64_t)(c0 + j) * sc];
+    return bitcast<raw_t>(r);
 }
-template <int DT>
+template <int DT, int CH>
 __device__ __forceinline__ void store_state_row(void *base, int64_t sb, int64_t sc, int64_t sl,
-                                                int b, int c0, int l, bool vec, const u32x4 &v) {
-    if (vec) {
-        st_vec<DT>(base, (int64_t)b * sb + (int64_t)l * sl + c0, v);
+                                                int b, int c0, int l,
+                                                const typename Pack<DT, CH>::raw_t &v) {
+    using T = typename Elem<DT>::type;
+    using raw_t = typename Pack<DT, CH>::raw_t;
+    T *row = reinterpret_cast<T *>(base) + (int64_t)b * sb + (int64_t)l * sl;
+    if (sc == 1 && (reinterpret_cast<uintptr_t>(row + c0) % sizeof(raw_t)) == 0) {
+        *reinterpret_cast<raw_t *>(row + c0) = v;
         return;
     }
-    RawVec<DT> r = bitcast<RawVec<DT>>(v);
+    const RawElems<DT, CH> r = bitcast<RawElems<DT, CH>>(v);
 #pragma unroll
-    for (int j = 0; j < Elem<DT>::kVec; ++j)
-        st_raw<DT>(base, (int64_t)b * sb + (int64_t)(c0 + j) * sc + (int64_t)l * sl, r.v[j]);
+    for (int j = 0; j < CH; ++j) row[(int64_t)(c0 + j) * sc] = r.v[j];
 }
 
-template <int DT, int W, bool HAS_SEQ, int U, bool NT>
-__global__ void __launch_bounds__(kBlock)
+template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U>
+__global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CC1D_FWD_CL_OCC8))
 fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     using E = Elem<DT>;
-    constexpr int VEC = E::kVec;
+    using T_ = typename E::type;
+    using P = Pack<DT, CH>;
+    using raw_t = typename P::raw_t;
     constexpr bool PRECISE = E::kPreciseAct;
 
-    const uint32_t gid = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
+    // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
+    const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
+    const uint32_t gid = block * (uint32_t)kBlock + threadIdx.x;
     if (gid >= g.total) return;                       // no cross-lane traffic below
     const uint32_t col = gid % (uint32_t)g.n_colgroups;
     const uint32_t rb = gid / (uint32_t)g.n_colgroups;
     const int run = (int)(rb % (uint32_t)g.n_runs);
     const int b = (int)(rb / (uint32_t)g.n_runs);
-    const int c0 = (int)col * VEC;
+    const int c0 = (int)col * CH;
     const int L = p.seqlen;
-    const int T = g.rows_per_run;
+    const int T = g.rows_per_run;                     // multiple of 2*U
     const int t0 = run * T;                           // < L by construction of n_runs
-    const bool silu_on = p.silu != 0;
+    const int last = L - 1 - t0;                      // last valid row of this run, run-relative
 
-    float wv[VEC][W], bv[VEC];
-    load_weights<W, VEC>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
-                         g.w_fast != 0, c0, wv, bv);
+    float wv[CH][W], bv[CH];
+    load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
+                        g.w_fast != 0, c0, wv, bv);
 
     const int64_t xoff = (int64_t)b * p.x_stride_b + c0;
     const int64_t ooff = (int64_t)b * p.out_stride_b + c0;
-    const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L : nullptr;
+    // Row pointers of this run; offsets inside a run fit 32 bits (checked by the launcher).
+    const char *xrun = reinterpret_cast<const char *>(reinterpret_cast<const T_ *>(p.x) + xoff + (int64_t)t0 * p.x_stride_l);
+    char *orun = reinterpret_cast<char *>(reinterpret_cast<T_ *>(p.out) + ooff + (int64_t)t0 * p.out_stride_l);
+    const uint32_t xs = (uint32_t)p.x_stride_l * (uint32_t)sizeof(T_);
+    const uint32_t os = (uint32_t)p.out_stride_l * (uint32_t)sizeof(T_);
+    const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
 
     // Sliding window: xw[i] holds row t-(W-1)+i while row t is being produced.
-    float xw[W - 1][VEC];
+    float xw[W - 1][CH];
     int sqw[W - 1];
 #pragma unroll
     for (int i = 0; i < W - 1; ++i) {
         const int t = t0 - (W - 1) + i;
-        u32x4 r = {0u, 0u, 0u, 0u};
+        raw_t r = P::zero();
         if (t >= 0) {
-            r = ld_vec<DT>(p.x, xoff + (int64_t)t * p.x_stride_l);
+            r = *reinterpret_cast<const raw_t *>(xrun - (int64_t)(W - 1 - i) * xs);
         } else if (p.initial_states != nullptr) {
-            r = load_state_row<DT>(p.initial_states, p.init_stride_b, p.init_stride_c,
-                                   p.init_stride_l, b, c0, t + (W - 1), g.init_vec != 0);
+            r = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
+                                       p.init_stride_l, b, c0, t + (W - 1));
         }
-        E::unpack(r, xw[i]);
-        sqw[i] = (HAS_SEQ && t >= 0) ? seq[t] : -1;
+        P::unpack(r, xw[i]);
+        // Rows in front of the sequence hold zeros unless initial_states are given; with
+        // zeros a mask changes nothing, so they take the first row's id and do not make
+        // the first group look like a boundary.
+        sqw[i] = !HAS_SEQ ? 0 : t >= 0 ? seq[i - (W - 1)] : p.initial_states != nullptr ? -1 : seq[-t0];
     }
 
-    u32x4 nraw[U];
-    int nseq[U];
-    auto load_group = [&](int t) {
+    // CHECKED = false: the whole run lies inside the sequence, so loads and stores are
+    // unconditional (the wait counts the compiler derives are then exact and loads stay
+    // in flight across stores).  CHECKED = true: the ragged last run of a sequence; rows
+    // past its end re-read the last valid row and their stores are suppressed.
+    // STREAM: non-temporal loads; the last rows of a run are read with the normal policy
+    // because the following run needs them again as its halo.
+    auto load_group = [&](auto checked, auto stream, int i0, raw_t (&raw)[U], int (&sq)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int tt = t + u;
-            u32x4 r = {0u, 0u, 0u, 0u};
-            int s = -1;
-            if (tt < L) {
-                r = NT ? ld_vec_nt<DT>(p.x, xoff + (int64_t)tt * p.x_stride_l)
-                       : ld_vec<DT>(p.x, xoff + (int64_t)tt * p.x_stride_l);
-                if (HAS_SEQ) s = seq[tt];
-            }
-            nraw[u] = r;
-            nseq[u] = s;
+            const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
+            const raw_t *src = reinterpret_cast<const raw_t *>(xrun + (uint32_t)i * xs);
+            raw[u] = decltype(stream)::value ? __builtin_nontemporal_load(src) : *src;
+            if (HAS_SEQ && (decltype(checked)::value || U % 4 != 0)) sq[u] = seq[i];
+            if (!HAS_SEQ) sq[u] = 0;
         }
-    };
-    load_group(t0);
-
-    for (int i = 0; i < T; i += U) {
-        u32x4 raw[U];
-        int sq[U];
+        if (HAS_SEQ && !decltype(checked)::value && U % 4 == 0) {
+            if (g.seq_vec) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) { raw[u] = nraw[u]; sq[u] = nseq[u]; }
-        if (i + U < T) load_group(t0 + i + U);        // prefetch the next group of rows
-
+                for (int q = 0; q < U / 4; ++q) {
+                    const u32x4 s4 = *reinterpret_cast<const u32x4 *>(seq + i0 + 4 * q);
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = t0 + i + u;
-            float xv[VEC], acc[VEC];
-            E::unpack(raw[u], xv);
-
-            bool plain = true;
-            if (HAS_SEQ) {
-                const int cur = sq[u];
-                plain = cur >= 0;
-#pragma unroll
-                for (int k = 0; k < W - 1; ++k) plain = plain && (sqw[k] == cur);
-            }
-            if (plain) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    float a = bv[j];
-#pragma unroll
-                    for (int k = 0; k < W - 1; ++k) a = fmaf(wv[j][k], xw[k][j], a);
-                    acc[j] = fmaf(wv[j][W - 1], xv[j], a);
+                    for (int k = 0; k < 4; ++k) sq[4 * q + k] = (int)s4[k];
                 }
             } else {
-                // A sub-sequence boundary (or padding) inside the window: rare, so the
-                // masked form lives on its own branch.
-                const int cur = sq[u];
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
+                for (int u = 0; u < U; ++u) sq[u] = seq[i0 + u];
+            }
+        }
+    };
+
+    // With seq_idx the walk computes every row as if no sub-sequence boundary were near
+    // (no branch in the hot loop) and only records, per lane, the span of row groups whose
+    // rows or window are not all of one non-negative id.  Those few rows are redone with
+    // masked taps after the walk.
+    int redo_lo = T, redo_hi = 0;
+    auto compute_group = [&](auto checked, int i0, const raw_t (&raw)[U], const int (&sq)[U]) {
+        if (HAS_SEQ) {
+            uint32_t lo = (uint32_t)sq[0], hi = (uint32_t)sq[0];
+#pragma unroll
+            for (int u = 1; u < U; ++u) { lo = min(lo, (uint32_t)sq[u]); hi = max(hi, (uint32_t)sq[u]); }
+#pragma unroll
+            for (int k = 0; k < W - 1; ++k) { lo = min(lo, (uint32_t)sqw[k]); hi = max(hi, (uint32_t)sqw[k]); }
+            if (lo != hi || (int)hi < 0) { redo_lo = min(redo_lo, i0); redo_hi = max(redo_hi, i0 + U); }
+#pragma unroll
+            for (int k = 0; k < W - 1; ++k) sqw[k] = sq[U - (W - 1) + k];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float xv[CH], acc[CH];
+            P::unpack(raw[u], xv);
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                float a = bv[j];
+#pragma unroll
+                for (int k = 0; k < W - 1; ++k) a = fmaf(wv[j][k], xw[k][j], a);
+                a = fmaf(wv[j][W - 1], xv[j], a);
+                acc[j] = SILU ? silu<PRECISE>(a) : a;
+            }
+            if (!decltype(checked)::value || i0 + u <= last)
+                __builtin_nontemporal_store(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
+#pragma unroll
+            for (int k = 0; k < W - 2; ++k)
+#pragma unroll
+                for (int j = 0; j < CH; ++j) xw[k][j] = xw[k + 1][j];
+#pragma unroll
+            for (int j = 0; j < CH; ++j) xw[W - 2][j] = xv[j];
+        }
+    };
+
+    using No = std::integral_constant<bool, false>;
+    using Yes = std::integral_constant<bool, true>;
+    static_assert(U >= W - 1, "a group must cover the window");
+    raw_t ra[U], rb_[U];
+    int sa[U], sb[U];
+    if (last >= T - 1) {
+        // Two register sets in ping-pong: while one group of U rows is computed and stored,
+        // the next two groups' loads are in flight, and nothing is copied at the loop edge
+        // (a copy would make the compiler wait for every outstanding access).  The first
+        // and the last pair of groups are peeled: the loop is then entered in exactly the
+        // state its back edge leaves (stores A, loads A, stores B, loads B pending), which
+        // keeps the compiler's wait counts exact, and no load sits behind an exit test.
+        if (T > 2 * U) {
+            load_group(No{}, Yes{}, 0, ra, sa);
+            load_group(No{}, Yes{}, U, rb_, sb);
+            compute_group(No{}, 0, ra, sa);
+            int i = 2 * U;
+            if (T > 4 * U) {
+                load_group(No{}, Yes{}, 2 * U, ra, sa);
+                compute_group(No{}, U, rb_, sb);
+                load_group(No{}, Yes{}, 3 * U, rb_, sb);
+#pragma clang loop unroll(disable)
+                for (; i + 4 * U < T; i += 2 * U) {
+                    compute_group(No{}, i, ra, sa);
+                    load_group(No{}, Yes{}, i + 2 * U, ra, sa);
+                    compute_group(No{}, i + U, rb_, sb);
+                    load_group(No{}, Yes{}, i + 3 * U, rb_, sb);
+                }
+                compute_group(No{}, i, ra, sa);
+                load_group(No{}, Yes{}, i + 2 * U, ra, sa);
+                compute_group(No{}, i + U, rb_, sb);
+                i += 2 * U;
+            } else {
+                load_group(No{}, Yes{}, 2 * U, ra, sa);
+                compute_group(No{}, U, rb_, sb);
+            }
+            load_group(No{}, No{}, i + U, rb_, sb);   // the run's last rows: keep them cached
+            compute_group(No{}, i, ra, sa);
+            compute_group(No{}, i + U, rb_, sb);
+        } else {
+            load_group(No{}, Yes{}, 0, ra, sa);
+            load_group(No{}, No{}, U, rb_, sb);
+            compute_group(No{}, 0, ra, sa);
+            compute_group(No{}, U, rb_, sb);
+        }
+    } else {
+        for (int i = 0; i <= last; i += U) {
+            load_group(Yes{}, No{}, i, ra, sa);
+            compute_group(Yes{}, i, ra, sa);
+        }
+    }
+
+    if (HAS_SEQ) {
+        // Rows near a sub-sequence boundary or in padding, one group of U rows per trip:
+        // taps masked row by row (csrc/causal_conv1d_fwd.cu:316-329), padding tokens exactly
+        // zero.  All U+W-1 rows and ids a group needs are requested at once, straight from
+        // memory (they were streamed moments ago), with no branch between the loads; the
+        // results overwrite what the walk stored for these rows.
+#pragma clang loop unroll(disable)
+        for (int i0 = redo_lo; i0 < redo_hi; i0 += U) {
+            float xr[U + W - 1][CH];
+            int sr[U + W - 1];
+#pragma unroll
+            for (int q = 0; q < U + W - 1; ++q) {
+                int i = i0 - (W - 1) + q;              // run-relative row of slot q
+                const bool before = t0 + i < 0;       // in front of the sequence: no data
+                i = i > last ? last : i;
+                i = before ? 0 : i;
+                P::unpack(*reinterpret_cast<const raw_t *>(xrun + (int64_t)i * xs), xr[q]);
+                const int id = seq[i];
+                sr[q] = before ? -1 : id;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int cur = sr[W - 1 + u];
+                float acc[CH];
+#pragma unroll
+                for (int j = 0; j < CH; ++j) {
                     float a = bv[j];
 #pragma unroll
                     for (int k = 0; k < W - 1; ++k)
-                        a = fmaf(sqw[k] == cur ? wv[j][k] : 0.f, xw[k][j], a);
-                    acc[j] = fmaf(wv[j][W - 1], xv[j], a);
+                        a = fmaf(sr[u + k] == cur ? wv[j][k] : 0.f, xr[u + k][j], a);
+                    a = fmaf(wv[j][W - 1], xr[u + W - 1][j], a);
+                    if (SILU) a = silu<PRECISE>(a);
+                    acc[j] = cur < 0 ? 0.f : a;
                 }
+                if (i0 + u <= last)
+                    __builtin_nontemporal_store(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
             }
-            if (silu_on) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = silu<PRECISE>(acc[j]);
-            }
-            if (HAS_SEQ) {
-                if (sq[u] < 0) {                      // padding token: exact zero
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-                }
-            }
-            if (t < L) {
-                const u32x4 o = E::pack(acc);
-                if (NT) st_vec_nt<DT>(p.out, ooff + (int64_t)t * p.out_stride_l, o);
-                else st_vec<DT>(p.out, ooff + (int64_t)t * p.out_stride_l, o);
-            }
-#pragma unroll
-            for (int k = 0; k < W - 2; ++k) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) xw[k][j] = xw[k + 1][j];
-                sqw[k] = sqw[k + 1];
-            }
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) xw[W - 2][j] = xv[j];
-            sqw[W - 2] = sq[u];
         }
     }
 
@@ -201,75 +307,85 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) {
             const int t = L - (W - 1) + i;
-            u32x4 r = {0u, 0u, 0u, 0u};
+            raw_t r = P::zero();
             if (t >= 0) {
-                r = ld_vec<DT>(p.x, xoff + (int64_t)t * p.x_stride_l);
+                r = *reinterpret_cast<const raw_t *>(reinterpret_cast<const T_ *>(p.x) + xoff + (int64_t)t * p.x_stride_l);
             } else if (p.initial_states != nullptr) {
-                r = load_state_row<DT>(p.initial_states, p.init_stride_b, p.init_stride_c,
-                                       p.init_stride_l, b, c0, t + (W - 1), g.init_vec != 0);
+                r = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
+                                           p.init_stride_l, b, c0, t + (W - 1));
             }
-            store_state_row<DT>(p.final_states, p.final_stride_b, p.final_stride_c,
-                                p.final_stride_l, b, c0, i, g.final_vec != 0, r);
+            store_state_row<DT, CH>(p.final_states, p.final_stride_b, p.final_stride_c,
+                                    p.final_stride_l, b, c0, i, r);
         }
     }
 }
 
-template <int DT, int W, bool HAS_SEQ>
+template <int DT, int CH, int W, bool HAS_SEQ>
 int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
-    const uint32_t blocks = (g.total + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL((fwd_channellast_kernel<DT, W, HAS_SEQ, CC1D_FWD_CL_UNROLL, CC1D_FWD_CL_NT != 0>),
-                       dim3(blocks), dim3(kBlock), 0, stream, p, g);
+    constexpr int U = CC1D_FWD_CL_UNROLL;
+    const uint32_t blocks = g.blocks_per_xcd * kXcds;
+    if (p.silu)
+        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>),
+                           dim3(blocks), dim3(kBlock), 0, stream, p, g);
+    else
+        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>),
+                           dim3(blocks), dim3(kBlock), 0, stream, p, g);
     return launch_status();
 }
 
-template <int DT>
-int launch_dtype(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
+template <int DT, int CH>
+int launch_width(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
     const bool seq = p.seq_idx != nullptr;
     switch (p.width) {
-        case 2: return seq ? launch_instance<DT, 2, true>(p, g, stream) : launch_instance<DT, 2, false>(p, g, stream);
-        case 3: return seq ? launch_instance<DT, 3, true>(p, g, stream) : launch_instance<DT, 3, false>(p, g, stream);
-        default: return seq ? launch_instance<DT, 4, true>(p, g, stream) : launch_instance<DT, 4, false>(p, g, stream);
+        case 2: return seq ? launch_instance<DT, CH, 2, true>(p, g, stream) : launch_instance<DT, CH, 2, false>(p, g, stream);
+        case 3: return seq ? launch_instance<DT, CH, 3, true>(p, g, stream) : launch_instance<DT, CH, 3, false>(p, g, stream);
+        default: return seq ? launch_instance<DT, CH, 4, true>(p, g, stream) : launch_instance<DT, CH, 4, false>(p, g, stream);
     }
 }
 
 }  // namespace
 
-// Rows walked by one lane.  Longer runs amortise the (W-1)-row halo re-read; shorter
-// runs put more wavefronts in flight.  The target is about 24 waves per CU on 256 CUs
-// while keeping the halo overhead at or below (W-1)/32.
-static int choose_rows_per_run(int64_t batch, int64_t n_colgroups, int seqlen) {
-    constexpr int U = CC1D_FWD_CL_UNROLL;
-    int forced = tunables().fwd_cl_rows;
-    int T;
-    if (forced > 0) {
-        T = forced;
-    } else {
-        const int64_t target_lanes = (int64_t)256 * 24 * kWave;
-        T = 128;
-        while (T > 32 && batch * n_colgroups * ((seqlen + T - 1) / T) < target_lanes) T >>= 1;
-    }
+// Rows walked by one lane.  Longer runs amortise the per-run start-up (taps, halo); shorter
+// runs put more wavefronts in flight, which is what keeps HBM busy while other waves
+// compute, and spread the work more evenly over the CUs.  32 rows measured best at the
+// prefill shape (8 x 2048 rows x 5376 channels); short sequences take what they have.
+static int choose_rows_per_run(int seqlen, int64_t row_bytes) {
+    constexpr int U = 2 * CC1D_FWD_CL_UNROLL;         // the walk is unrolled over two groups
+    int T = tunables().fwd_cl_rows;
+    if (T <= 0) T = 32;
     const int cap = (seqlen + U - 1) / U * U;          // never longer than the sequence
     if (T > cap) T = cap;
     T = (T + U - 1) / U * U;
-    return T < U ? U : T;
+    if (T < U) T = U;
+    // Byte offsets inside a run are 32-bit in the kernel.
+    while (T > U && (int64_t)T * row_bytes >= ((int64_t)1 << 31)) T = (T / 2 + U - 1) / U * U;
+    return (int64_t)T * row_bytes >= ((int64_t)1 << 31) ? 0 : T;
 }
 
 int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
-    const int vec = vec_elems(p.x_dtype);
+    // Channels per lane: an 8-byte vector (4 x 16-bit or 2 x fp32).  Half the registers of a
+    // 16-byte lane, so twice the waves per SIMD to overlap compute with memory; measured
+    // 9% faster at the prefill shape.  fwd_cl_half_vec = -1 selects 16-byte lanes.
+    const int full = vec_elems(p.x_dtype);
+    const int ch = tunables().fwd_cl_half_vec < 0 ? full : full / 2;
     FwdClGeom g;
-    g.n_colgroups = p.dim / vec;
-    g.rows_per_run = choose_rows_per_run(p.batch, g.n_colgroups, p.seqlen);
+    g.n_colgroups = p.dim / ch;
+    const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
+    g.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * elem_bytes(p.x_dtype));
+    if (g.rows_per_run == 0) return CC1D_ERR_TOO_LARGE;
     g.n_runs = (p.seqlen + g.rows_per_run - 1) / g.rows_per_run;
     const int64_t total = (int64_t)p.batch * g.n_runs * g.n_colgroups;
-    if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+    if (total >= ((int64_t)1 << 31) - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
     g.total = (uint32_t)total;
+    const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
+    g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
-    g.init_vec = states_vec_ok(p.initial_states, p.x_dtype, p.init_stride_b, p.init_stride_c, p.init_stride_l);
-    g.final_vec = states_vec_ok(p.final_states, p.x_dtype, p.final_stride_b, p.final_stride_c, p.final_stride_l);
+    g.seq_vec = p.seq_idx != nullptr && p.seqlen % 4 == 0 && aligned16(p.seq_idx);
+    const bool half = ch != full;
     switch (p.x_dtype) {
-        case CC1D_F32: return launch_dtype<CC1D_F32>(p, g, stream);
-        case CC1D_F16: return launch_dtype<CC1D_F16>(p, g, stream);
-        default: return launch_dtype<CC1D_BF16>(p, g, stream);
+        case CC1D_F32: return half ? launch_width<CC1D_F32, 2>(p, g, stream) : launch_width<CC1D_F32, 4>(p, g, stream);
+        case CC1D_F16: return half ? launch_width<CC1D_F16, 4>(p, g, stream) : launch_width<CC1D_F16, 8>(p, g, stream);
+        default: return half ? launch_width<CC1D_BF16, 4>(p, g, stream) : launch_width<CC1D_BF16, 8>(p, g, stream);
     }
 }
 

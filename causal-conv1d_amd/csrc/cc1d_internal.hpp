@@ -37,6 +37,7 @@ inline bool states_vec_ok(const void *p, int x_dtype, int64_t sb, int64_t sc, in
 
 struct Tunables {
     int32_t fwd_cl_rows = 0;
+    int32_t fwd_cl_half_vec = 0;
     int32_t bwd_cl_rows = 0;
     int32_t fwd_cf_vecs = 0;
     int32_t bwd_cf_parts = 0;

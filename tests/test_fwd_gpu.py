@@ -145,22 +145,36 @@ def test_fwd_chunking_is_bit_exact_at_prefill_size(pkg, gpu_device):
     assert torch.equal(pkg.causal_conv1d_fn(x, w, b, seq_idx=torch.zeros_like(seq), activation="silu"), whole)
 
 
-def test_fwd_rows_per_run_does_not_change_results(pkg, gpu_device, cc1d_lib):
-    """Every run length of the channel-last walk gives the same bits."""
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fwd_launch_geometry_does_not_change_results(pkg, gpu_device, cc1d_lib, dtype):
+    """Every run length and both lane widths (16- and 8-byte vectors) of the channel-last
+    walk give the same bits, with seq_idx, padding, initial and final states."""
     lib = cabi.declare(cc1d_lib)
     g = gen(11)
-    x = make_x(2, 264, 333, torch.bfloat16, True, g).to(gpu_device)
+    x = make_x(2, 264, 333, dtype, True, g).to(gpu_device)
     w, b = (t.to(gpu_device) for t in make_wb(264, 4, True, g))
-    seq = random_seq_idx(2, 333, g).to(gpu_device)
+    seq = random_seq_idx(2, 333, g, pad=True).to(gpu_device)
+    init = make_states(2, 264, 3, dtype, g).to(gpu_device)
     outs = []
     try:
-        for rows in (4, 8, 32, 64, 128, 1024):
-            assert lib.cc1d_set_tunable(b"fwd_cl_rows", rows) == 0
-            outs.append(pkg.causal_conv1d_fn(x, w, b, seq_idx=seq, activation="silu").cpu())
+        for half in (0, -1):
+            for rows in (8, 16, 32, 64, 128, 1024):
+                assert lib.cc1d_set_tunable(b"fwd_cl_rows", rows) == 0
+                assert lib.cc1d_set_tunable(b"fwd_cl_half_vec", half) == 0
+                o1 = pkg.causal_conv1d_fn(x, w, b, seq_idx=seq, activation="silu")
+                o2, f2 = pkg.causal_conv1d_fn(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+                outs.append((o1.cpu(), o2.cpu(), f2.cpu()))
     finally:
         lib.cc1d_set_tunable(b"fwd_cl_rows", 0)
+        lib.cc1d_set_tunable(b"fwd_cl_half_vec", 0)
     for o in outs[1:]:
-        assert torch.equal(o, outs[0])
+        for a, r in zip(o, outs[0]):
+            assert torch.equal(a, r)
+    xc = x.cpu()
+    assert_close(outs[0][0], orc.fwd_seq_idx(xc, w.cpu(), b.cpu(), seq.cpu(), activation="silu"), dtype, "seq_idx")
+    ref, fin = orc.fwd(xc, w.cpu(), b.cpu(), initial_states=init.cpu(), return_final_states=True, activation="silu")
+    assert_close(outs[0][1], ref, dtype, "states")
+    assert torch.equal(outs[0][2], fin)
 
 
 def test_fwd_through_the_c_abi_on_a_side_stream(gpu_device, cc1d_lib):
