@@ -24,14 +24,14 @@
 
 // Rows per register set; two sets are in flight per lane.
 #ifndef CC1D_FWD_CL_UNROLL
-#define CC1D_FWD_CL_UNROLL 4
+#define CC1D_FWD_CL_UNROLL 8
 #endif
 // Workgroups per CU the register budget must allow, for 16- and 8-byte lanes.
 #ifndef CC1D_FWD_CL_OCC16
 #define CC1D_FWD_CL_OCC16 2
 #endif
 #ifndef CC1D_FWD_CL_OCC8
-#define CC1D_FWD_CL_OCC8 4
+#define CC1D_FWD_CL_OCC8 3
 #endif
 
 namespace cc1d {
