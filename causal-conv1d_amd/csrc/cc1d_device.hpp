@@ -317,6 +317,14 @@ __device__ __forceinline__ float silu(float z) {
         return z * sigmoid<false>(z);
     }
 }
+// SiLU of z given y = -log2(e) * z (the caller folds that factor into the taps and the bias,
+// which saves one multiply per element):  z sigmoid(z) = y / (c + c 2^y),  c = -log2(e).
+__device__ __forceinline__ float silu_from_scaled(float y) {
+    constexpr float c = -1.4426950408889634f;
+    return y * __builtin_amdgcn_rcpf(fmaf(__builtin_amdgcn_exp2f(y), c, c));
+}
+constexpr float kSiluPrescale = -1.4426950408889634f;
+
 // d silu(z) / dz = s (1 + z (1 - s)),  s = sigmoid(z)  (csrc/causal_conv1d_bwd.cu:168-170)
 template <bool PRECISE>
 __device__ __forceinline__ float silu_grad(float z) {

@@ -110,6 +110,17 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     float wv[CH][W], bv[CH];
     load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
                         g.w_fast != 0, c0, wv, bv);
+    // 16-bit outputs with SiLU: taps and bias carry the factor -log2(e), so the sums below
+    // are already the exponent the activation needs (see silu_from_scaled).
+    constexpr bool SCALED = SILU && !PRECISE;
+    if (SCALED) {
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            bv[j] *= kSiluPrescale;
+#pragma unroll
+            for (int k = 0; k < W; ++k) wv[j][k] *= kSiluPrescale;
+        }
+    }
 
     const int64_t xoff = (int64_t)b * p.x_stride_b + c0;
     const int64_t ooff = (int64_t)b * p.out_stride_b + c0;
@@ -196,7 +207,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
 #pragma unroll
                 for (int k = 0; k < W - 1; ++k) a = fmaf(wv[j][k], xw[k][j], a);
                 a = fmaf(wv[j][W - 1], xv[j], a);
-                acc[j] = SILU ? silu<PRECISE>(a) : a;
+                acc[j] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
             }
             if (!decltype(checked)::value || i0 + u <= last)
                 __builtin_nontemporal_store(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
@@ -292,7 +303,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
                     for (int k = 0; k < W - 1; ++k)
                         a = fmaf(sr[u + k] == cur ? wv[j][k] : 0.f, xr[u + k][j], a);
                     a = fmaf(wv[j][W - 1], xr[u + W - 1][j], a);
-                    if (SILU) a = silu<PRECISE>(a);
+                    if (SILU) a = SCALED ? silu_from_scaled(a) : silu<PRECISE>(a);
                     acc[j] = cur < 0 ? 0.f : a;
                 }
                 if (i0 + u <= last)
