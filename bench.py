@@ -294,8 +294,8 @@ def cpu_baseline(cfg_cpu, n_bytes):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--rows", type=int, default=0, help="override rows per lane run (sweeps)")
