@@ -9,347 +9,454 @@
 //   dweight[w] += sum_{b,t} g[t] * xpad[t-(W-1-w)],   dbias += sum_{b,t} g[t]
 // with every tap additionally masked by seq_idx equality when seq_idx is given.
 //
-// Design.  Same geometry as the channel-last forward: a lane owns one 16-byte vector of
-// channels and walks a run of rows in ascending order, holding (W-1)-row sliding windows
-// of x and g in registers.  dx[p] is emitted W-1 steps late, when g[p+W-1] has arrived,
-// so one ascending pass yields dx, and the lane's dweight/dbias partial sums stay in
-// registers for the whole run (no cross-lane reduction, no atomics).  Each run then
-// stores its partials to a workspace plane and a second kernel adds them up in a fixed
-// order: results are bit-reproducible.  Halo cost per run: W-1 rows of x in front,
-// W-1 rows of x and dout behind.
+// Design.  Same geometry as the channel-last forward: a lane owns CH adjacent channels
+// (one 8-byte vector) and walks a run of T rows in ascending order, holding (W-1)-row
+// sliding windows of x and g in registers.  The run owns g[t] (hence the dweight/dbias
+// terms) for its rows t in [t0, t1) and emits dx one window late: row t completes
+// dx[t-(W-1)], so the run writes dx[t0-(W-1) .. t1-(W-1)).  Everything a run needs from
+// its neighbour is therefore in front of it (2(W-1) rows of x, W-1 rows of dout, loaded
+// once before the walk and found in L2, see the forward kernel), and the walk itself is
+// uniform: two loads, one store and the same arithmetic for every row, no branch.  The last
+// run of a sequence adds the W-1 closing rows, run 0 routes rows in front of the sequence
+// to dinitial_states.  A lane's dweight/dbias partial sums stay in registers for the whole
+// run (no cross-lane reduction, no atomics); each run stores them to a workspace plane and
+// a second kernel adds the planes up in a fixed order: results are bit-reproducible.
+#include <type_traits>
+
 #include "cc1d_device.hpp"
 #include "cc1d_internal.hpp"
 
+// Rows per register set; two sets are in flight per lane.
 #ifndef CC1D_BWD_CL_UNROLL
-#define CC1D_BWD_CL_UNROLL 2
+#define CC1D_BWD_CL_UNROLL 4
+#endif
+// Workgroups per CU the register budget must allow.
+#ifndef CC1D_BWD_CL_OCC
+#define CC1D_BWD_CL_OCC 2
 #endif
 
 namespace cc1d {
 namespace {
 
+constexpr int kXcds = 8;
+
 struct BwdClGeom {
-    int32_t rows_per_run;
-    int32_t n_runs;
-    int32_t n_colgroups;
-    uint32_t total;
-    int32_t w_fast;
-    int32_t init_vec;
-    int32_t dinit_vec;
+    int32_t rows_per_run;     // T, a multiple of twice the unroll factor
+    int32_t n_runs;           // ceil(seqlen / T)
+    int32_t n_colgroups;      // dim / CH
+    uint32_t total;           // batch * n_runs * n_colgroups work items
+    uint32_t blocks_per_xcd;  // grid size / 8
+    int32_t w_fast;           // weights_contiguous_f32
 };
 
-template <int DT>
-struct alignas(16) RawVecB {
-    typename Elem<DT>::type v[Elem<DT>::kVec];
-};
-
-template <int DT, int W, bool HAS_SEQ, bool SILU, int U>
-__global__ void __launch_bounds__(kBlock)
+template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U>
+__global__ void __launch_bounds__(kBlock, CC1D_BWD_CL_OCC)
 bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws) {
     using E = Elem<DT>;
-    constexpr int VEC = E::kVec;
+    using T_ = typename E::type;
+    using P = Pack<DT, CH>;
+    using raw_t = typename P::raw_t;
     constexpr bool PRECISE = E::kPreciseAct;
 
-    const uint32_t gid = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
-    if (gid >= g.total) return;
+    // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
+    const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
+    const uint32_t gid = block * (uint32_t)kBlock + threadIdx.x;
+    if (gid >= g.total) return;                       // no cross-lane traffic below
     const uint32_t col = gid % (uint32_t)g.n_colgroups;
     const uint32_t rb = gid / (uint32_t)g.n_colgroups;
     const int run = (int)(rb % (uint32_t)g.n_runs);
     const int b = (int)(rb / (uint32_t)g.n_runs);
-    const int c0 = (int)col * VEC;
+    const int c0 = (int)col * CH;
     const int L = p.seqlen;
     const int T = g.rows_per_run;
-    const int t0 = run * T;
-    const int t1 = t0 + T < L ? t0 + T : L;           // rows [t0, t1) are this lane's own
-    const int t_last = t1 + (W - 1);                  // exclusive end of the walk
+    const int t0 = run * T;                           // < L by construction of n_runs
+    const bool full = t0 + T <= L;                    // the run lies inside the sequence
+    const int last = full ? T - 1 : L - 1 - t0;       // last row of this run, run-relative
 
-    float wv[VEC][W], bv[VEC];
-    load_weights<W, VEC>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
-                         g.w_fast != 0, c0, wv, bv);
+    float wv[CH][W], bv[CH];
+    load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
+                        g.w_fast != 0, c0, wv, bv);
 
-    const int64_t xoff = (int64_t)b * p.x_stride_b + c0;
-    const int64_t doff = (int64_t)b * p.dout_stride_b + c0;
-    const int64_t dxoff = (int64_t)b * p.dx_stride_b + c0;
-    const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L : nullptr;
+    // Row pointers of this run; offsets inside a run fit 32 bits (checked by the launcher).
+    const char *xrun = reinterpret_cast<const char *>(reinterpret_cast<const T_ *>(p.x) + (int64_t)b * p.x_stride_b + c0 + (int64_t)t0 * p.x_stride_l);
+    const char *drun = reinterpret_cast<const char *>(reinterpret_cast<const T_ *>(p.dout) + (int64_t)b * p.dout_stride_b + c0 + (int64_t)t0 * p.dout_stride_l);
+    // Row i of the walk stores dx row i-(W-1): the pointer is moved back once instead.
+    char *dxrun = reinterpret_cast<char *>(reinterpret_cast<T_ *>(p.dx) + (int64_t)b * p.dx_stride_b + c0) +
+                  ((int64_t)t0 - (W - 1)) * p.dx_stride_l * (int64_t)sizeof(T_);
+    const uint32_t xs = (uint32_t)p.x_stride_l * (uint32_t)sizeof(T_);
+    const uint32_t ds = (uint32_t)p.dout_stride_l * (uint32_t)sizeof(T_);
+    const uint32_t dxs = (uint32_t)p.dx_stride_l * (uint32_t)sizeof(T_);
+    const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
 
-    // Windows: xw[k] = x[t-(W-1)+k], gw[k] = g[t-(W-1)+k], sqw[k] likewise, at step t.
-    float xw[W - 1][VEC], gw[W - 1][VEC];
-    int sqw[W - 1];
+    // g[t] = dout[t] * act'(z[t]) from the x window in front of row t; taps that cross a
+    // sub-sequence boundary are masked, padding rows (id < 0) have no gradient.
+    auto grad_row = [&](const float (&xwin)[W - 1][CH], const int (&idwin)[W - 1], const float (&xv)[CH],
+                        int cur, float (&gv)[CH]) {
+        if (SILU) {
 #pragma unroll
-    for (int k = 0; k < W - 1; ++k) {
-        const int t = t0 - (W - 1) + k;
-        u32x4 r = {0u, 0u, 0u, 0u};
-        if (t >= 0) {
-            r = ld_vec<DT>(p.x, xoff + (int64_t)t * p.x_stride_l);
-        } else if (p.initial_states != nullptr) {
-            if (g.init_vec) {
-                r = ld_vec<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
-                                                     (int64_t)(t + W - 1) * p.init_stride_l + c0);
-            } else {
-                RawVecB<DT> rv;
+            for (int j = 0; j < CH; ++j) {
+                float z = bv[j];
 #pragma unroll
-                for (int j = 0; j < VEC; ++j)
-                    rv.v[j] = ld_raw<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
-                                                               (int64_t)(c0 + j) * p.init_stride_c +
-                                                               (int64_t)(t + W - 1) * p.init_stride_l);
-                r = bitcast<u32x4>(rv);
+                for (int k = 0; k < W - 1; ++k)
+                    z = fmaf((!HAS_SEQ || idwin[k] == cur) ? xwin[k][j] : 0.f, wv[j][k], z);
+                z = fmaf(wv[j][W - 1], xv[j], z);
+                gv[j] *= silu_grad<PRECISE>(z);
             }
         }
-        E::unpack(r, xw[k]);
+        if (HAS_SEQ) {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) gw[k][j] = 0.f;
-        sqw[k] = (HAS_SEQ && t >= 0) ? seq[t] : -1;
+            for (int j = 0; j < CH; ++j) gv[j] = cur < 0 ? 0.f : gv[j];
+        }
+    };
+    // dx[pp] = sum_k weight[W-1-k] * g[pp+k]; gwin holds g[pp .. pp+W-2], gv is g[pp+W-1].
+    auto dx_row = [&](const float (&gwin)[W - 1][CH], const int (&idwin)[W - 1], const float (&gv)[CH],
+                      int cur, float (&dxv)[CH]) {
+        const int sp = idwin[0];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            float a = wv[j][W - 1] * gwin[0][j];
+#pragma unroll
+            for (int k = 1; k < W - 1; ++k)
+                a = fmaf((!HAS_SEQ || idwin[k] == sp) ? gwin[k][j] : 0.f, wv[j][W - 1 - k], a);
+            a = fmaf((!HAS_SEQ || cur == sp) ? gv[j] : 0.f, wv[j][0], a);
+            dxv[j] = a;
+        }
+    };
+
+    // Windows at row t: xw[k] = x[t-(W-1)+k], gw[k] = g[t-(W-1)+k], sqw[k] the ids.
+    // Filling gw needs the x rows and ids another W-1 steps back.
+    float xw[W - 1][CH], gw[W - 1][CH];
+    int sqw[W - 1];
+    {
+        float xh[2 * (W - 1)][CH];
+        int sh[2 * (W - 1)];
+        raw_t dh[W - 1];
+#pragma unroll
+        for (int q = 0; q < 2 * (W - 1); ++q) {
+            const int t = t0 - 2 * (W - 1) + q;
+            raw_t r = P::zero();
+            if (t >= 0) {
+                r = *reinterpret_cast<const raw_t *>(xrun - (int64_t)(2 * (W - 1) - q) * xs);
+            } else if (p.initial_states != nullptr && t >= -(W - 1)) {
+                r = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
+                                           p.init_stride_l, b, c0, t + (W - 1));
+            }
+            P::unpack(r, xh[q]);
+            sh[q] = (HAS_SEQ && t >= 0) ? seq[q - 2 * (W - 1)] : -1;
+        }
+#pragma unroll
+        for (int k = 0; k < W - 1; ++k) {
+            const int t = t0 - (W - 1) + k;
+            dh[k] = P::zero();
+            if (t >= 0) dh[k] = *reinterpret_cast<const raw_t *>(drun - (int64_t)(W - 1 - k) * ds);
+        }
+#pragma unroll
+        for (int k = 0; k < W - 1; ++k) {
+            float xwin[W - 1][CH];
+            int idwin[W - 1];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) {
+                idwin[i] = sh[k + i];
+#pragma unroll
+                for (int j = 0; j < CH; ++j) xwin[i][j] = xh[k + i][j];
+            }
+            P::unpack(dh[k], gw[k]);                  // zero in front of the sequence
+            grad_row(xwin, idwin, xh[k + W - 1], sh[k + W - 1], gw[k]);
+#pragma unroll
+            for (int j = 0; j < CH; ++j) xw[k][j] = xh[k + W - 1][j];
+            sqw[k] = sh[k + W - 1];
+        }
     }
 
-    float dW[VEC][W], dB[VEC];
+    float dW[CH][W], dB[CH];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
+    for (int j = 0; j < CH; ++j) {
         dB[j] = 0.f;
 #pragma unroll
         for (int w = 0; w < W; ++w) dW[j][w] = 0.f;
     }
 
-    u32x4 nx[U], nd[U];
-    int nseq[U];
-    auto load_group = [&](int t) {
+    // CHECKED = false: loads and stores are unconditional (the wait counts the compiler
+    // derives are then exact and loads stay in flight across stores).  CHECKED = true: the
+    // first rows of run 0 (positions in front of the sequence go to dinitial_states) and
+    // ragged or short runs (rows past the end re-read the last valid row and are inert).
+    // STREAM: non-temporal loads; the last rows of a run are read with the normal policy
+    // because the following run needs them again as its halo.
+    auto load_group = [&](auto checked, auto stream, int i0, raw_t (&rx)[U], raw_t (&rd)[U], int (&sq)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int tt = t + u;
-            u32x4 rx = {0u, 0u, 0u, 0u}, rd = {0u, 0u, 0u, 0u};
-            int s = -1;
-            if (tt < L && tt < t_last) {
-                rx = ld_vec_nt<DT>(p.x, xoff + (int64_t)tt * p.x_stride_l);
-                rd = ld_vec_nt<DT>(p.dout, doff + (int64_t)tt * p.dout_stride_l);
-                if (HAS_SEQ) s = seq[tt];
-            }
-            nx[u] = rx; nd[u] = rd; nseq[u] = s;
+            const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
+            const raw_t *sx = reinterpret_cast<const raw_t *>(xrun + (uint32_t)i * xs);
+            const raw_t *sd = reinterpret_cast<const raw_t *>(drun + (uint32_t)i * ds);
+            rx[u] = decltype(stream)::value ? __builtin_nontemporal_load(sx) : *sx;
+            rd[u] = decltype(stream)::value ? __builtin_nontemporal_load(sd) : *sd;
+            sq[u] = HAS_SEQ ? seq[i] : 0;
         }
     };
-    load_group(t0);
-
-    const int n_steps = T + (W - 1);                  // uniform trip count; extra steps are inert
-    for (int i = 0; i < n_steps; i += U) {
-        u32x4 rx[U], rd[U];
-        int sq[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) { rx[u] = nx[u]; rd[u] = nd[u]; sq[u] = nseq[u]; }
-        if (i + U < n_steps) load_group(t0 + i + U);
-
+    auto compute_group = [&](auto checked, int i0, const raw_t (&rx)[U], const raw_t (&rd)[U], const int (&sq)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int t = t0 + i + u;
+            if (decltype(checked)::value && i0 + u > last) continue;   // past the end: inert
             const int cur = sq[u];
-            float xv[VEC], gv[VEC];
-            E::unpack(rx[u], xv);
-            E::unpack(rd[u], gv);                     // dout[t]; zero for t >= L
-
-            bool tapm[W - 1];                         // tap k (row t-(W-1)+k) feeds row t
+            float xv[CH], gv[CH], dxv[CH];
+            P::unpack(rx[u], xv);
+            P::unpack(rd[u], gv);
+            grad_row(xw, sqw, xv, cur, gv);
 #pragma unroll
-            for (int k = 0; k < W - 1; ++k) tapm[k] = !HAS_SEQ || sqw[k] == cur;
-
-            if (SILU) {
+            for (int j = 0; j < CH; ++j) {
+                dB[j] += gv[j];
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    float z = bv[j];
-#pragma unroll
-                    for (int k = 0; k < W - 1; ++k) z = fmaf(tapm[k] ? wv[j][k] : 0.f, xw[k][j], z);
-                    z = fmaf(wv[j][W - 1], xv[j], z);
-                    gv[j] *= silu_grad<PRECISE>(z);
+                for (int k = 0; k < W - 1; ++k)
+                    dW[j][k] = fmaf(gv[j], (!HAS_SEQ || sqw[k] == cur) ? xw[k][j] : 0.f, dW[j][k]);
+                dW[j][W - 1] = fmaf(gv[j], xv[j], dW[j][W - 1]);
+            }
+            dx_row(gw, sqw, gv, cur, dxv);
+            if (!decltype(checked)::value) {
+                __builtin_nontemporal_store(P::pack(dxv), reinterpret_cast<raw_t *>(dxrun + (uint32_t)(i0 + u) * dxs));
+            } else {
+                // Row t < L completes position pp = t-(W-1) < L-(W-1): no dfinal term yet.
+                const int pp = t0 + i0 + u - (W - 1);
+                if (pp >= 0) {
+                    *reinterpret_cast<raw_t *>(dxrun + (int64_t)(i0 + u) * dxs) = P::pack(dxv);
+                } else if (p.dinitial_states != nullptr) {
+                    store_state_row<DT, CH>(p.dinitial_states, p.dinit_stride_b, p.dinit_stride_c,
+                                            p.dinit_stride_l, b, c0, pp + (W - 1), P::pack(dxv));
                 }
             }
-            if (HAS_SEQ) {
-                if (cur < 0) {
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j) gv[j] = 0.f;
-                }
-            }
-
-            if (t < t1) {                             // own row: dweight / dbias partials
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    dB[j] += gv[j];
-#pragma unroll
-                    for (int k = 0; k < W - 1; ++k)
-                        dW[j][k] = fmaf(gv[j], tapm[k] ? xw[k][j] : 0.f, dW[j][k]);
-                    dW[j][W - 1] = fmaf(gv[j], xv[j], dW[j][W - 1]);
-                }
-            }
-
-            // Emit position pp = t-(W-1): g[pp .. pp+W-2] = gw[0..W-2], g[pp+W-1] = gv.
-            const int pp = t - (W - 1);
-            const bool emit_dx = pp >= t0 && pp < t1;
-            const bool emit_dinit = pp < 0 && t0 == 0 && p.dinitial_states != nullptr && t < W - 1;
-            if (emit_dx || emit_dinit) {
-                const int sp = sqw[0];
-                float dxv[VEC];
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    float a = wv[j][W - 1] * gw[0][j];
-#pragma unroll
-                    for (int k = 1; k < W - 1; ++k)
-                        a = fmaf((!HAS_SEQ || sqw[k] == sp) ? wv[j][W - 1 - k] : 0.f, gw[k][j], a);
-                    a = fmaf((!HAS_SEQ || cur == sp) ? wv[j][0] : 0.f, gv[j], a);
-                    dxv[j] = a;
-                }
-                if (p.dfinal_states != nullptr && pp >= L - (W - 1)) {
-                    const int fl = pp - (L - (W - 1));
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        dxv[j] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
-                                                                   (int64_t)(c0 + j) * p.dfinal_stride_c +
-                                                                   (int64_t)fl * p.dfinal_stride_l);
-                }
-                if (emit_dx) {
-                    st_vec_nt<DT>(p.dx, dxoff + (int64_t)pp * p.dx_stride_l, E::pack(dxv));
-                } else {
-                    const int il = pp + (W - 1);
-                    if (g.dinit_vec) {
-                        st_vec<DT>(p.dinitial_states, (int64_t)b * p.dinit_stride_b +
-                                                          (int64_t)il * p.dinit_stride_l + c0, E::pack(dxv));
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j)
-                            st_elem<DT>(p.dinitial_states, (int64_t)b * p.dinit_stride_b +
-                                                               (int64_t)(c0 + j) * p.dinit_stride_c +
-                                                               (int64_t)il * p.dinit_stride_l, dxv[j]);
-                    }
-                }
-            }
-
 #pragma unroll
             for (int k = 0; k < W - 2; ++k) {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) { xw[k][j] = xw[k + 1][j]; gw[k][j] = gw[k + 1][j]; }
+                for (int j = 0; j < CH; ++j) { xw[k][j] = xw[k + 1][j]; gw[k][j] = gw[k + 1][j]; }
                 sqw[k] = sqw[k + 1];
             }
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) { xw[W - 2][j] = xv[j]; gw[W - 2][j] = gv[j]; }
+            for (int j = 0; j < CH; ++j) { xw[W - 2][j] = xv[j]; gw[W - 2][j] = gv[j]; }
             sqw[W - 2] = cur;
+        }
+    };
+
+    using No = std::integral_constant<bool, false>;
+    using Yes = std::integral_constant<bool, true>;
+    // Run 0 routes positions in front of the sequence through the checked form of its first
+    // group only, so that group must hold all W-1 of them.
+    static_assert(U >= W - 1, "the first group must cover the window");
+    raw_t xa[U], da[U], xb[U], db[U];
+    int sa[U], sb[U];
+    if (full && T >= 6 * U) {
+        // Two register sets in ping-pong: while one group of U rows is computed and stored,
+        // the loads of the next two groups are in flight, and nothing is copied at the loop
+        // edge.  The first and the last pair of groups are peeled, so the loop is entered
+        // in exactly the state its back edge leaves and the wait counts stay exact.
+        load_group(No{}, Yes{}, 0, xa, da, sa);
+        load_group(No{}, Yes{}, U, xb, db, sb);
+        if (run > 0) compute_group(No{}, 0, xa, da, sa);
+        else compute_group(Yes{}, 0, xa, da, sa);     // rows in front of the sequence: dinitial_states
+        load_group(No{}, Yes{}, 2 * U, xa, da, sa);
+        compute_group(No{}, U, xb, db, sb);
+        load_group(No{}, Yes{}, 3 * U, xb, db, sb);
+        int i = 2 * U;
+#pragma clang loop unroll(disable)
+        for (; i + 4 * U < T; i += 2 * U) {
+            compute_group(No{}, i, xa, da, sa);
+            load_group(No{}, Yes{}, i + 2 * U, xa, da, sa);
+            compute_group(No{}, i + U, xb, db, sb);
+            load_group(No{}, Yes{}, i + 3 * U, xb, db, sb);
+        }
+        // i + 4U == T: the run's last 2U rows stay cached for the next run's halo.
+        compute_group(No{}, i, xa, da, sa);
+        load_group(No{}, No{}, i + 2 * U, xa, da, sa);
+        compute_group(No{}, i + U, xb, db, sb);
+        load_group(No{}, No{}, i + 3 * U, xb, db, sb);
+        compute_group(No{}, i + 2 * U, xa, da, sa);
+        compute_group(No{}, i + 3 * U, xb, db, sb);
+    } else {
+        for (int i = 0; i <= last; i += U) {
+            load_group(Yes{}, No{}, i, xa, da, sa);
+            compute_group(Yes{}, i, xa, da, sa);
         }
     }
 
-    // Partials of this run: plane w of part (b, run), channels c0 .. c0+VEC.
+    // The sequence's last run closes it: dx[L-(W-1) .. L) see no further g (zero past the
+    // end) and take dfinal_states; with seqlen < W-1 part of that lands in dinitial_states
+    // (csrc/causal_conv1d_bwd.cu:535-541, 555-559).
+    if (run == g.n_runs - 1) {
+        float zero[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) zero[j] = 0.f;
+#pragma unroll
+        for (int k = 0; k < W - 1; ++k) {
+            const int pp = L - (W - 1) + k;
+            float dxv[CH];
+            dx_row(gw, sqw, zero, -1, dxv);
+            if (p.dfinal_states != nullptr) {
+                const raw_t fr = load_state_row<DT, CH>(p.dfinal_states, p.dfinal_stride_b, p.dfinal_stride_c,
+                                                        p.dfinal_stride_l, b, c0, k);
+                float fv[CH];
+                P::unpack(fr, fv);
+#pragma unroll
+                for (int j = 0; j < CH; ++j) dxv[j] += fv[j];
+            }
+            if (pp >= 0) {
+                *reinterpret_cast<raw_t *>(reinterpret_cast<T_ *>(p.dx) + (int64_t)b * p.dx_stride_b + c0 +
+                                           (int64_t)pp * p.dx_stride_l) = P::pack(dxv);
+            } else if (p.dinitial_states != nullptr) {
+                store_state_row<DT, CH>(p.dinitial_states, p.dinit_stride_b, p.dinit_stride_c,
+                                        p.dinit_stride_l, b, c0, pp + (W - 1), P::pack(dxv));
+            }
+#pragma unroll
+            for (int q = 0; q < W - 2; ++q) {
+#pragma unroll
+                for (int j = 0; j < CH; ++j) gw[q][j] = gw[q + 1][j];
+                sqw[q] = sqw[q + 1];
+            }
+#pragma unroll
+            for (int j = 0; j < CH; ++j) gw[W - 2][j] = 0.f;
+            sqw[W - 2] = -1;
+        }
+    }
+
+    // Partials of this run: plane w of part (b, run), channels c0 .. c0+CH.
     const int64_t part = (int64_t)b * g.n_runs + run;
     float *dst = ws + part * (int64_t)(W + 1) * p.dim + c0;
 #pragma unroll
     for (int w = 0; w <= W; ++w) {
+        typename RawBytes<CH * 4>::type o;
 #pragma unroll
-        for (int q = 0; q < VEC / 4; ++q) {
-            u32x4 o;
-            if (w < W) {
-                o.x = bitcast<uint32_t>(dW[4 * q][w]); o.y = bitcast<uint32_t>(dW[4 * q + 1][w]);
-                o.z = bitcast<uint32_t>(dW[4 * q + 2][w]); o.w = bitcast<uint32_t>(dW[4 * q + 3][w]);
-            } else {
-                o.x = bitcast<uint32_t>(dB[4 * q]); o.y = bitcast<uint32_t>(dB[4 * q + 1]);
-                o.z = bitcast<uint32_t>(dB[4 * q + 2]); o.w = bitcast<uint32_t>(dB[4 * q + 3]);
-            }
-            *reinterpret_cast<u32x4 *>(dst + (int64_t)w * p.dim + 4 * q) = o;
-        }
+        for (int j = 0; j < CH; ++j) o[j] = bitcast<uint32_t>(w < W ? dW[j][w] : dB[j]);
+        *reinterpret_cast<typename RawBytes<CH * 4>::type *>(dst + (int64_t)w * p.dim) = o;
     }
 }
 
 }  // namespace
 
-// Second stage shared by both backward layouts: dweight[c, w] += sum over parts, in
-// ascending part order, of ws[part][w][c]; plane W holds dbias.  One lane per (w, c).
-__global__ void __launch_bounds__(kBlock)
+// Second stage shared by both backward layouts: dweight[c, w] += sum over parts of
+// ws[part][w][c]; plane W holds dbias.  A workgroup owns 64 channels of one plane; its 16
+// wavefronts each add up every 16th part (four independent chains, so the loads overlap),
+// and wavefront 0 combines the 16 slice sums through LDS.  The order of the additions is a
+// function of n_parts alone, so results are bit-reproducible.
+constexpr int kFinSlices = 16;
+constexpr int kFinChannels = 64;
+
+__global__ void __launch_bounds__(kFinSlices * kFinChannels)
 bwd_finalize_kernel(const float *__restrict__ ws, int n_parts, int dim, int width,
                     float *__restrict__ dweight, int64_t dw_stride_c, int64_t dw_stride_w,
                     float *__restrict__ dbias) {
-    const uint32_t gid = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
-    const uint32_t planes = (uint32_t)width + (dbias != nullptr ? 1u : 0u);
-    if (gid >= planes * (uint32_t)dim) return;
-    const int c = (int)(gid % (uint32_t)dim);
-    const int w = (int)(gid / (uint32_t)dim);
+    __shared__ float slice_sum[kFinSlices][kFinChannels];
+    const int lane = (int)threadIdx.x % kFinChannels;
+    const int slice = (int)threadIdx.x / kFinChannels;
+    const int cblocks = (dim + kFinChannels - 1) / kFinChannels;
+    const int w = (int)blockIdx.x / cblocks;
+    const int c = ((int)blockIdx.x % cblocks) * kFinChannels + lane;
     const int64_t part_stride = (int64_t)(width + 1) * dim;
-    const float *src = ws + (int64_t)w * dim + c;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;    // four interleaved chains, fixed order
-    int q = 0;
-    for (; q + 4 <= n_parts; q += 4) {
-        s0 += src[(int64_t)q * part_stride];
-        s1 += src[(int64_t)(q + 1) * part_stride];
-        s2 += src[(int64_t)(q + 2) * part_stride];
-        s3 += src[(int64_t)(q + 3) * part_stride];
+    float s = 0.f;
+    if (c < dim) {
+        const float *src = ws + (int64_t)w * dim + c;
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        int q = slice;
+        for (; q + 3 * kFinSlices < n_parts; q += 4 * kFinSlices) {
+            s0 += src[(int64_t)q * part_stride];
+            s1 += src[(int64_t)(q + kFinSlices) * part_stride];
+            s2 += src[(int64_t)(q + 2 * kFinSlices) * part_stride];
+            s3 += src[(int64_t)(q + 3 * kFinSlices) * part_stride];
+        }
+        for (; q < n_parts; q += kFinSlices) s0 += src[(int64_t)q * part_stride];
+        s = (s0 + s1) + (s2 + s3);
     }
-    for (; q < n_parts; ++q) s0 += src[(int64_t)q * part_stride];
-    const float total = (s0 + s1) + (s2 + s3);
-    if (w < width) dweight[(int64_t)c * dw_stride_c + (int64_t)w * dw_stride_w] += total;
-    else dbias[c] += total;
+    slice_sum[slice][lane] = s;
+    __syncthreads();
+    if (slice == 0 && c < dim) {
+        float total = 0.f;
+#pragma unroll
+        for (int i = 0; i < kFinSlices; ++i) total += slice_sum[i][lane];
+        if (w < width) dweight[(int64_t)c * dw_stride_c + (int64_t)w * dw_stride_w] += total;
+        else dbias[c] += total;
+    }
 }
 
 int launch_bwd_finalize(const float *ws, int n_parts, const cc1d_bwd_params &p, hipStream_t stream) {
     const uint32_t planes = (uint32_t)p.width + (p.dbias != nullptr ? 1u : 0u);
-    const uint32_t total = planes * (uint32_t)p.dim;
-    hipLaunchKernelGGL(bwd_finalize_kernel, dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
+    const uint32_t cblocks = ((uint32_t)p.dim + kFinChannels - 1) / kFinChannels;
+    hipLaunchKernelGGL(bwd_finalize_kernel, dim3(planes * cblocks), dim3(kFinSlices * kFinChannels), 0, stream,
                        ws, n_parts, p.dim, p.width, p.dweight, p.dw_stride_c, p.dw_stride_w, p.dbias);
     return launch_status();
 }
 
 namespace {
 
-BwdClGeom make_geom(const cc1d_bwd_params &p) {
-    constexpr int U = CC1D_BWD_CL_UNROLL;
-    const int vec = vec_elems(p.x_dtype);
-    BwdClGeom g;
-    g.n_colgroups = p.dim / vec;
+int channels_per_lane(int x_dtype) { return vec_elems(x_dtype) / 2; }   // 8-byte lanes
+
+// Returns false when a run cannot be addressed with 32-bit byte offsets.
+bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
+    constexpr int U2 = 2 * CC1D_BWD_CL_UNROLL;        // the walk is unrolled over two groups
+    g.n_colgroups = p.dim / channels_per_lane(p.x_dtype);
     int T = tunables().bwd_cl_rows;
+    // Runs of 128 rows: the halo in front of a run and its partial-sum planes then cost about
+    // 5% of the tensor traffic while the prefill shape still launches 2688 wavefronts; measured
+    // best against 32, 64 and 256 there.
     if (T <= 0) {
-        // Runs of 128 rows keep the partial-sum planes at about 2.6% of the tensor traffic;
-        // go shorter only when that is needed to put about 8 waves on each of 256 CUs.
-        const int64_t target_lanes = (int64_t)256 * 8 * kWave;
         T = 128;
+        // Small problems: shorter runs until about 8 wavefronts per CU exist.
+        const int64_t target_lanes = (int64_t)256 * 8 * kWave;
         while (T > 32 && (int64_t)p.batch * g.n_colgroups * ((p.seqlen + T - 1) / T) < target_lanes) T >>= 1;
     }
-    const int cap = (p.seqlen + U - 1) / U * U;
+    const int cap = (p.seqlen + U2 - 1) / U2 * U2;     // never longer than the sequence
     if (T > cap) T = cap;
-    T = (T + U - 1) / U * U;
-    if (T < U) T = U;
+    T = (T + U2 - 1) / U2 * U2;
+    if (T < U2) T = U2;
+    int64_t row_stride = p.x_stride_l > p.dout_stride_l ? p.x_stride_l : p.dout_stride_l;
+    if (p.dx_stride_l > row_stride) row_stride = p.dx_stride_l;
+    const int64_t row_bytes = row_stride * elem_bytes(p.x_dtype);
+    while (T > U2 && (int64_t)(T + U2) * row_bytes >= ((int64_t)1 << 31)) T = (T / 2 + U2 - 1) / U2 * U2;
+    if ((int64_t)(T + U2) * row_bytes >= ((int64_t)1 << 31)) return false;
     g.rows_per_run = T;
     g.n_runs = (p.seqlen + T - 1) / T;
-    g.total = 0;
+    const int64_t total = (int64_t)p.batch * g.n_runs * g.n_colgroups;
+    if (total >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
+    g.total = (uint32_t)total;
+    const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
+    g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
-    g.init_vec = states_vec_ok(p.initial_states, p.x_dtype, p.init_stride_b, p.init_stride_c, p.init_stride_l);
-    g.dinit_vec = states_vec_ok(p.dinitial_states, p.x_dtype, p.dinit_stride_b, p.dinit_stride_c, p.dinit_stride_l);
-    return g;
+    return true;
 }
 
-template <int DT, int W, bool HAS_SEQ>
+template <int DT, int CH, int W, bool HAS_SEQ>
 int launch_instance(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStream_t stream) {
-    const uint32_t blocks = (g.total + kBlock - 1) / kBlock;
+    constexpr int U = CC1D_BWD_CL_UNROLL;
+    const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, W, HAS_SEQ, true, CC1D_BWD_CL_UNROLL>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws);
+        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws);
     else
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, W, HAS_SEQ, false, CC1D_BWD_CL_UNROLL>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws);
+        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws);
     return launch_status();
 }
 
-template <int DT>
+template <int DT, int CH>
 int launch_dtype(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStream_t stream) {
     const bool seq = p.seq_idx != nullptr;
     switch (p.width) {
-        case 2: return seq ? launch_instance<DT, 2, true>(p, g, ws, stream) : launch_instance<DT, 2, false>(p, g, ws, stream);
-        case 3: return seq ? launch_instance<DT, 3, true>(p, g, ws, stream) : launch_instance<DT, 3, false>(p, g, ws, stream);
-        default: return seq ? launch_instance<DT, 4, true>(p, g, ws, stream) : launch_instance<DT, 4, false>(p, g, ws, stream);
+        case 2: return seq ? launch_instance<DT, CH, 2, true>(p, g, ws, stream) : launch_instance<DT, CH, 2, false>(p, g, ws, stream);
+        case 3: return seq ? launch_instance<DT, CH, 3, true>(p, g, ws, stream) : launch_instance<DT, CH, 3, false>(p, g, ws, stream);
+        default: return seq ? launch_instance<DT, CH, 4, true>(p, g, ws, stream) : launch_instance<DT, CH, 4, false>(p, g, ws, stream);
     }
 }
 
 }  // namespace
 
 size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p) {
-    const BwdClGeom g = make_geom(p);
+    BwdClGeom g;
+    if (!make_geom(p, g)) return 0;
     return (size_t)p.batch * g.n_runs * (p.width + 1) * (size_t)p.dim * sizeof(float);
 }
 
 int launch_bwd_channellast(const cc1d_bwd_params &p, void *workspace, hipStream_t stream) {
-    BwdClGeom g = make_geom(p);
-    const int64_t total = (int64_t)p.batch * g.n_runs * g.n_colgroups;
-    if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
-    g.total = (uint32_t)total;
+    BwdClGeom g;
+    if (!make_geom(p, g)) return CC1D_ERR_TOO_LARGE;
     float *ws = static_cast<float *>(workspace);
     int st;
     switch (p.x_dtype) {
-        case CC1D_F32: st = launch_dtype<CC1D_F32>(p, g, ws, stream); break;
-        case CC1D_F16: st = launch_dtype<CC1D_F16>(p, g, ws, stream); break;
-        default: st = launch_dtype<CC1D_BF16>(p, g, ws, stream); break;
+        case CC1D_F32: st = launch_dtype<CC1D_F32, 2>(p, g, ws, stream); break;
+        case CC1D_F16: st = launch_dtype<CC1D_F16, 4>(p, g, ws, stream); break;
+        default: st = launch_dtype<CC1D_BF16, 4>(p, g, ws, stream); break;
     }
     if (st != CC1D_OK) return st;
     return launch_bwd_finalize(ws, p.batch * g.n_runs, p, stream);

@@ -332,4 +332,39 @@ __device__ __forceinline__ float silu_grad(float z) {
     return s * (1.0f + z * (1.0f - s));
 }
 
+template <int DT, int CH>
+struct alignas(CH * Elem<DT>::kBytes) RawElems {
+    typename Elem<DT>::type v[CH];
+};
+
+// CH channels of one (batch, l) row of a (batch, dim, k) states tensor.
+template <int DT, int CH>
+__device__ __forceinline__ typename Pack<DT, CH>::raw_t
+load_state_row(const void *base, int64_t sb, int64_t sc, int64_t sl, int b, int c0, int l) {
+    using T = typename Elem<DT>::type;
+    using raw_t = typename Pack<DT, CH>::raw_t;
+    const T *row = reinterpret_cast<const T *>(base) + (int64_t)b * sb + (int64_t)l * sl;
+    if (sc == 1 && (reinterpret_cast<uintptr_t>(row + c0) % sizeof(raw_t)) == 0)
+        return *reinterpret_cast<const raw_t *>(row + c0);
+    RawElems<DT, CH> r;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) r.v[j] = row[(int64_t)(c0 + j) * sc];
+    return bitcast<raw_t>(r);
+}
+template <int DT, int CH>
+__device__ __forceinline__ void store_state_row(void *base, int64_t sb, int64_t sc, int64_t sl,
+                                                int b, int c0, int l,
+                                                const typename Pack<DT, CH>::raw_t &v) {
+    using T = typename Elem<DT>::type;
+    using raw_t = typename Pack<DT, CH>::raw_t;
+    T *row = reinterpret_cast<T *>(base) + (int64_t)b * sb + (int64_t)l * sl;
+    if (sc == 1 && (reinterpret_cast<uintptr_t>(row + c0) % sizeof(raw_t)) == 0) {
+        *reinterpret_cast<raw_t *>(row + c0) = v;
+        return;
+    }
+    const RawElems<DT, CH> r = bitcast<RawElems<DT, CH>>(v);
+#pragma unroll
+    for (int j = 0; j < CH; ++j) row[(int64_t)(c0 + j) * sc] = r.v[j];
+}
+
 }  // namespace cc1d
