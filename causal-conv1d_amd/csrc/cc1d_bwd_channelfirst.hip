@@ -18,6 +18,14 @@
 // Only an item's first and last step fall back to a few wave-uniform element loads.
 // Rows of x, dout and dx may sit on different 16-byte grids; lanes follow x's grid and
 // the other tensors use vectors when they share it, elements otherwise.
+//
+// Two kernels share this design.  The streaming kernel takes rows that are 16-byte aligned
+// and whose length is a whole number of step pairs (every power-of-two seqlen from 1024
+// up): no bounds checks, two register sets in ping-pong, and lane 0's x halo is a separate
+// small load of its own, so the sets do not depend on each other and the loads of the next
+// two steps stay in flight while a step is computed.  The general kernel takes the rest.
+#include <type_traits>
+
 #include "cc1d_device.hpp"
 #include "cc1d_internal.hpp"
 
@@ -25,6 +33,7 @@ namespace cc1d {
 namespace {
 
 struct BwdCfGeom {
+    int32_t streaming;        // aligned rows, whole step pairs: the streaming kernel applies
     int32_t vecs_per_seg;     // multiple of 64
     int32_t n_segs;           // segments per row
     int32_t n_items;          // batch * n_segs
@@ -289,6 +298,205 @@ bwd_channelfirst_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__res
     }
 }
 
+template <int DT, int W>
+__global__ void __launch_bounds__(kBlock)
+bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__restrict__ ws) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    constexpr int VEC = E::kVec;
+    constexpr bool PRECISE = E::kPreciseAct;
+    // The four elements in front of a step, as one aligned load: 8 bytes of 16-bit data or
+    // 16 bytes of fp32; the last W-1 of them are lane 0's halo.
+    constexpr int HALO = 4;
+    using halo_t = typename RawBytes<HALO * E::kBytes>::type;
+    using HP = Pack<DT, HALO>;
+
+    const uint32_t wid = (blockIdx.x * (uint32_t)kBlock + threadIdx.x) / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    if (wid >= (uint32_t)p.dim * (uint32_t)g.n_parts) return;     // whole wave leaves together
+    const int part = (int)(wid % (uint32_t)g.n_parts);
+    const int c = (int)(wid / (uint32_t)g.n_parts);
+    const int L = p.seqlen;
+
+    RowCtx<DT, W> rc{p};
+    rc.c = c;
+    rc.silu_on = p.silu != 0;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+        rc.wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
+    rc.bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+
+    float dW[W], dB = 0.f;
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = 0.f;
+
+    const int item_begin = part * g.items_per_part;
+    int item_end = item_begin + g.items_per_part;
+    if (item_end > g.n_items) item_end = g.n_items;
+    const int n_vecs = L / VEC;
+
+    using No = std::integral_constant<bool, false>;
+    using Yes = std::integral_constant<bool, true>;
+
+    for (int item = item_begin; item < item_end; ++item) {
+        const int seg = item % g.n_segs;
+        const int b = item / g.n_segs;
+        rc.b = b;
+        rc.xrow = (int64_t)b * p.x_stride_b + (int64_t)c * p.x_stride_c;
+        rc.drow = (int64_t)b * p.dout_stride_b + (int64_t)c * p.dout_stride_c;
+        const T *xr = reinterpret_cast<const T *>(p.x) + rc.xrow;
+        const T *dr = reinterpret_cast<const T *>(p.dout) + rc.drow;
+        T *dxr = reinterpret_cast<T *>(p.dx) + (int64_t)b * p.dx_stride_b + (int64_t)c * p.dx_stride_c;
+
+        const int j_begin = seg * g.vecs_per_seg;
+        int j_end = j_begin + g.vecs_per_seg;
+        if (j_end > n_vecs) j_end = n_vecs;
+        const int n_steps = (j_end - j_begin) / kWave;            // even, >= 2 (or 0)
+        if (n_steps <= 0) continue;
+        const bool row_top = j_end == n_vecs, row_bottom = j_begin == 0;
+
+        // g just right of the item: zero past the row's end, else the next segment's first
+        // positions, recomputed from memory.
+        float carry_g[W - 1];
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i) carry_g[i] = row_top ? 0.f : rc.g_at(j_end * VEC + i);
+
+        // Step k counts down the row: k = 0 is the item's highest 64 vectors.
+        auto load_step = [&](int k, u32x4 &rx, u32x4 &rd, halo_t &rh) {
+            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;   // first element of the step
+            rx = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xr + e0 + lane * VEC));
+            rd = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(dr + e0 + lane * VEC));
+            const int h0 = e0 >= HALO ? e0 - HALO : 0;              // row start: replaced below
+            rh = *reinterpret_cast<const halo_t *>(xr + h0);
+        };
+        auto compute_step = [&](auto top, auto bottom, int k, const u32x4 &rx, const u32x4 &rd, const halo_t &rh) {
+            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;
+            float xf[VEC], gf[VEC], hf[HALO], carry_x[W - 1];
+            E::unpack(rx, xf);
+            E::unpack(rd, gf);
+            HP::unpack(rh, hf);
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) carry_x[i] = hf[HALO - (W - 1) + i];
+            if (decltype(bottom)::value) {
+                if (row_bottom) {
+#pragma unroll
+                    for (int i = 0; i < W - 1; ++i) carry_x[i] = rc.x_at(i - (W - 1));
+                }
+            }
+            // xx[i] = xpad at position tf-(W-1)+i
+            float xx[VEC + W - 1];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry_x[i]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xf[e];
+            if (rc.silu_on) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float z = rc.bias_v;
+#pragma unroll
+                    for (int w = 0; w < W; ++w) z = fmaf(rc.wv[w], xx[e + w], z);
+                    gf[e] *= silu_grad<PRECISE>(z);
+                }
+            }
+            // gg[i] = g at position tf+i, i in [0, VEC+W-1)
+            float gg[VEC + W - 1];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) gg[e] = gf[e];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) {
+                gg[VEC + i] = from_next_lane(gf[i], carry_g[i]);
+                carry_g[i] = read_lane(gf[i], 0);
+            }
+            float dxv[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float a = 0.f;
+#pragma unroll
+                for (int k2 = 0; k2 < W; ++k2) a = fmaf(rc.wv[W - 1 - k2], gg[e + k2], a);
+                dxv[e] = a;
+            }
+            if (decltype(top)::value) {
+                if (row_top && p.dfinal_states != nullptr && lane == kWave - 1) {
+#pragma unroll
+                    for (int i = 0; i < W - 1; ++i)
+                        dxv[VEC - (W - 1) + i] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
+                                                                               (int64_t)c * p.dfinal_stride_c +
+                                                                               (int64_t)i * p.dfinal_stride_l);
+                }
+            }
+            __builtin_nontemporal_store(E::pack(dxv), reinterpret_cast<u32x4 *>(dxr + e0 + lane * VEC));
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                dB += gf[e];
+#pragma unroll
+                for (int w = 0; w < W; ++w) dW[w] = fmaf(gf[e], xx[e + w], dW[w]);
+            }
+            if (decltype(bottom)::value) {
+                // dinitial_states[i] = dx at position i-(W-1) < 0: only g[0 .. i] reach it.
+                if (row_bottom && p.dinitial_states != nullptr && lane == 0) {
+#pragma unroll
+                    for (int i = 0; i < W - 1; ++i) {
+                        float a = 0.f;
+#pragma unroll
+                        for (int q = 0; q <= i; ++q) a = fmaf(rc.wv[i - q], gf[q], a);
+                        st_elem<DT>(p.dinitial_states, (int64_t)b * p.dinit_stride_b + (int64_t)c * p.dinit_stride_c +
+                                                           (int64_t)i * p.dinit_stride_l, a);
+                    }
+                }
+            }
+        };
+
+        // Two register sets in ping-pong; the first and last pair of steps are peeled so the
+        // loop is entered in the state its back edge leaves and the wait counts stay exact.
+        u32x4 ax, ad, bx, bd;
+        halo_t ah, bh;
+        load_step(0, ax, ad, ah);
+        load_step(1, bx, bd, bh);
+        if (n_steps == 2) {
+            compute_step(Yes{}, No{}, 0, ax, ad, ah);
+            compute_step(No{}, Yes{}, 1, bx, bd, bh);
+        } else {
+            compute_step(Yes{}, No{}, 0, ax, ad, ah);
+            load_step(2, ax, ad, ah);
+            compute_step(No{}, No{}, 1, bx, bd, bh);
+            load_step(3, bx, bd, bh);
+            int k = 2;
+#pragma clang loop unroll(disable)
+            for (; k + 2 < n_steps; k += 2) {
+                compute_step(No{}, No{}, k, ax, ad, ah);
+                load_step(k + 2, ax, ad, ah);
+                compute_step(No{}, No{}, k + 1, bx, bd, bh);
+                load_step(k + 3, bx, bd, bh);
+            }
+            compute_step(No{}, No{}, k, ax, ad, ah);
+            compute_step(No{}, Yes{}, k + 1, bx, bd, bh);
+        }
+    }
+
+    // One fixed-order reduction over the wave, then a single writer.
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = wave_sum(dW[w]);
+    dB = wave_sum(dB);
+    if (lane == 0) {
+        if (g.n_parts == 1) {
+#pragma unroll
+            for (int w = 0; w < W; ++w)
+                p.dweight[(int64_t)c * p.dw_stride_c + (int64_t)w * p.dw_stride_w] += dW[w];
+            if (p.dbias != nullptr) p.dbias[c] += dB;
+        } else {
+            float *dst = ws + (int64_t)part * (W + 1) * p.dim + c;
+#pragma unroll
+            for (int w = 0; w < W; ++w) dst[(int64_t)w * p.dim] = dW[w];
+            dst[(int64_t)W * p.dim] = dB;
+        }
+    }
+}
+
+// Rows of one tensor all start on a 16-byte boundary.
+bool rows_aligned(const void *base, int64_t stride_b, int64_t stride_c, int vec) {
+    return aligned16(base) && stride_b % vec == 0 && stride_c % vec == 0;
+}
+
 BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
     const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
@@ -299,11 +507,18 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int64_t max_parts = (int64_t)p.batch * max_steps;
     if (parts > max_parts) parts = max_parts;
     if (parts < 1) parts = 1;
+    const bool streaming = p.seqlen % (2 * kWave * vec) == 0 &&
+                           rows_aligned(p.x, p.x_stride_b, p.x_stride_c, vec) &&
+                           rows_aligned(p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
+                           rows_aligned(p.dx, p.dx_stride_b, p.dx_stride_c, vec);
     // Split rows into segments only if there are fewer rows per channel than slices.
     int64_t n_segs = (parts + p.batch - 1) / p.batch;
-    int64_t vps = (max_steps + n_segs - 1) / n_segs * kWave;
+    int64_t steps_per_seg = (max_steps + n_segs - 1) / n_segs;
+    if (streaming) steps_per_seg = (steps_per_seg + 1) / 2 * 2;    // whole step pairs
+    int64_t vps = steps_per_seg * kWave;
     n_segs = (max_vecs + vps - 1) / vps;
     BwdCfGeom g;
+    g.streaming = streaming ? 1 : 0;
     g.vecs_per_seg = (int32_t)vps;
     g.n_segs = (int32_t)n_segs;
     g.n_items = (int32_t)(p.batch * n_segs);
@@ -317,6 +532,14 @@ int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStr
     const int64_t waves = (int64_t)p.dim * g.n_parts;
     if (waves >= ((int64_t)1 << 25)) return CC1D_ERR_TOO_LARGE;
     const uint32_t blocks = (uint32_t)((waves + (kBlock / kWave) - 1) / (kBlock / kWave));
+    if (g.streaming) {
+        switch (p.width) {
+            case 2: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        }
+        return launch_status();
+    }
     switch (p.width) {
         case 2: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         case 3: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
