@@ -499,7 +499,12 @@ bool rows_aligned(const void *base, int64_t stride_b, int64_t stride_c, int vec)
 
 BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
-    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
+    const bool streaming = p.seqlen % (2 * kWave * vec) == 0 &&
+                           rows_aligned(p.x, p.x_stride_b, p.x_stride_c, vec) &&
+                           rows_aligned(p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
+                           rows_aligned(p.dx, p.dx_stride_b, p.dx_stride_c, vec);
+    // Worst case over row alignments: a row may start up to vec-1 elements into its grid.
+    const int64_t max_vecs = streaming ? p.seqlen / vec : ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
     const int64_t max_steps = (max_vecs + kWave - 1) / kWave;     // 64-vector steps per row
     // About 16 waves on each of 256 CUs when the problem allows it.
     int64_t parts = tunables().bwd_cf_parts > 0 ? tunables().bwd_cf_parts
@@ -507,10 +512,6 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int64_t max_parts = (int64_t)p.batch * max_steps;
     if (parts > max_parts) parts = max_parts;
     if (parts < 1) parts = 1;
-    const bool streaming = p.seqlen % (2 * kWave * vec) == 0 &&
-                           rows_aligned(p.x, p.x_stride_b, p.x_stride_c, vec) &&
-                           rows_aligned(p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
-                           rows_aligned(p.dx, p.dx_stride_b, p.dx_stride_c, vec);
     // Split rows into segments only if there are fewer rows per channel than slices.
     int64_t n_segs = (parts + p.batch - 1) / p.batch;
     int64_t steps_per_seg = (max_steps + n_segs - 1) / n_segs;

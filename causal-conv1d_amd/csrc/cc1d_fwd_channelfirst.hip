@@ -15,6 +15,14 @@
 // the same holds for `out` when its rows sit on a different grid than x's.
 // initial_states / final_states are supported (the reference refuses them for this
 // layout, csrc/causal_conv1d.cpp:213,228).
+//
+// Two kernels share this design.  The streaming kernel takes rows of x and out that are
+// 16-byte aligned and a whole number of step pairs long (every power-of-two seqlen from
+// 1024 up): no bounds checks, and two register sets in ping-pong keep the loads of the next
+// two steps in flight while a step is computed and stored.  The general kernel takes the
+// rest.
+#include <type_traits>
+
 #include "cc1d_device.hpp"
 #include "cc1d_internal.hpp"
 
@@ -22,6 +30,7 @@ namespace cc1d {
 namespace {
 
 struct FwdCfGeom {
+    int32_t streaming;        // steps per register set of the streaming kernel (1 or 2); 0: general kernel
     int32_t vecs_per_seg;     // multiple of 64
     int32_t n_segs;           // segments per row
     uint32_t total_waves;     // batch * dim * n_segs
@@ -151,8 +160,137 @@ fwd_channelfirst_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
     }
 }
 
+template <int DT, int W, bool SILU, int U>
+__global__ void __launch_bounds__(kBlock)
+fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    constexpr int VEC = E::kVec;
+    constexpr bool PRECISE = E::kPreciseAct;
+    // 16-bit outputs with SiLU: taps and bias carry the factor -log2(e), so the sums are
+    // already the exponent the activation needs (see silu_from_scaled).
+    constexpr bool SCALED = SILU && !PRECISE;
+
+    const uint32_t wid = (blockIdx.x * (uint32_t)kBlock + threadIdx.x) / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    if (wid >= g.total_waves) return;                 // whole wave leaves together
+    const int seg = (int)(wid % (uint32_t)g.n_segs);
+    const uint32_t row = wid / (uint32_t)g.n_segs;
+    const int c = (int)(row % (uint32_t)p.dim);
+    const int b = (int)(row / (uint32_t)p.dim);
+    const int L = p.seqlen;
+
+    const int64_t xrow = (int64_t)b * p.x_stride_b + (int64_t)c * p.x_stride_c;
+    const T *xr = reinterpret_cast<const T *>(p.x) + xrow;
+    T *orow = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b + (int64_t)c * p.out_stride_c;
+
+    const int n_vecs = L / VEC;
+    const int j_begin = seg * g.vecs_per_seg;
+    int j_end = j_begin + g.vecs_per_seg;
+    if (j_end > n_vecs) j_end = n_vecs;
+    const int n_groups = (j_end - j_begin) / (kWave * U);   // groups of U steps: even, >= 2 (or 0)
+
+    if (n_groups > 0) {
+        float wv[W], bias_v;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+            wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
+        bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+        if (SCALED) {
+            bias_v *= kSiluPrescale;
+#pragma unroll
+            for (int w = 0; w < W; ++w) wv[w] *= kSiluPrescale;
+        }
+
+        // Halo of the segment's first vector, wave-uniform.
+        float carry[W - 1];
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i)
+            carry[i] = padded_elem<DT, W>(p, xrow, b, c, j_begin * VEC - (W - 1) + i);
+
+        const T *xs = xr + (j_begin + lane) * VEC;    // this lane's vector of step 0
+        T *os = orow + (j_begin + lane) * VEC;
+        auto load_group = [&](int k, u32x4 (&raw)[U]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                raw[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xs + (k * U + u) * (kWave * VEC)));
+        };
+        auto compute_group = [&](int k, const u32x4 (&raw)[U]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float xf[VEC];
+                E::unpack(raw[u], xf);
+                // xx[i] = padded x at position tf - (W-1) + i
+                float xx[VEC + W - 1];
+#pragma unroll
+                for (int i = 0; i < W - 1; ++i) {
+                    xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry[i]);
+                    carry[i] = read_lane(xf[VEC - (W - 1) + i], kWave - 1);
+                }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xf[e];
+                float acc[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float a = bias_v;
+#pragma unroll
+                    for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
+                    acc[e] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
+                }
+                __builtin_nontemporal_store(E::pack(acc), reinterpret_cast<u32x4 *>(os + (k * U + u) * (kWave * VEC)));
+            }
+        };
+
+        // Two register sets of U steps in ping-pong; the first and last pair of groups are
+        // peeled so the loop is entered in the state its back edge leaves and the wait counts
+        // stay exact.
+        u32x4 ra[U], rb[U];
+        load_group(0, ra);
+        load_group(1, rb);
+        if (n_groups == 2) {
+            compute_group(0, ra);
+            compute_group(1, rb);
+        } else {
+            compute_group(0, ra);
+            load_group(2, ra);
+            compute_group(1, rb);
+            load_group(3, rb);
+            int k = 2;
+#pragma clang loop unroll(disable)
+            for (; k + 2 < n_groups; k += 2) {
+                compute_group(k, ra);
+                load_group(k + 2, ra);
+                compute_group(k + 1, rb);
+                load_group(k + 3, rb);
+            }
+            compute_group(k, ra);
+            compute_group(k + 1, rb);
+        }
+    }
+
+    // final_states[b, c, i] = xpad[L-(W-1)+i], bit-exact copies, by the row's first wave.
+    if (p.final_states != nullptr && seg == 0 && lane < W - 1) {
+        const int t = L - (W - 1) + lane;             // >= 0: a streaming row is at least 512 long
+        st_raw<DT>(p.final_states, (int64_t)b * p.final_stride_b + (int64_t)c * p.final_stride_c +
+                                       (int64_t)lane * p.final_stride_l, ld_raw<DT>(p.x, xrow + t));
+    }
+}
+
+template <int DT, bool SILU, int U>
+int launch_stream(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t stream) {
+    const uint32_t blocks = (g.total_waves + (kBlock / kWave) - 1) / (kBlock / kWave);
+    switch (p.width) {
+        case 2: hipLaunchKernelGGL((fwd_channelfirst_stream_kernel<DT, 2, SILU, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        case 3: hipLaunchKernelGGL((fwd_channelfirst_stream_kernel<DT, 3, SILU, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        default: hipLaunchKernelGGL((fwd_channelfirst_stream_kernel<DT, 4, SILU, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+    }
+    return launch_status();
+}
+
 template <int DT>
 int launch_dtype(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t stream) {
+    if (g.streaming == 2) return p.silu ? launch_stream<DT, true, 2>(p, g, stream) : launch_stream<DT, false, 2>(p, g, stream);
+    if (g.streaming == 1) return p.silu ? launch_stream<DT, true, 1>(p, g, stream) : launch_stream<DT, false, 1>(p, g, stream);
     const uint32_t blocks = (g.total_waves + (kBlock / kWave) - 1) / (kBlock / kWave);
     switch (p.width) {
         case 2: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
@@ -166,8 +304,12 @@ int launch_dtype(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t strea
 
 int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     const int vec = vec_elems(p.x_dtype);
+    const bool aligned = aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
+                         aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
+    // Steps per register set: two when rows split into whole pairs of two-step groups.
+    const int streaming = !aligned ? 0 : p.seqlen % (4 * kWave * vec) == 0 ? 2 : p.seqlen % (2 * kWave * vec) == 0 ? 1 : 0;
     // Worst case over row alignments: a row may start up to vec-1 elements into its grid.
-    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
+    const int64_t max_vecs = streaming ? p.seqlen / vec : ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
     const int64_t rows = (int64_t)p.batch * p.dim;
     int64_t vps;
     if (tunables().fwd_cf_vecs > 0) {
@@ -177,9 +319,11 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
         const int64_t want_segs = rows >= 4096 ? 1 : (4096 + rows - 1) / rows;
         vps = (max_vecs + want_segs - 1) / want_segs;
     }
-    vps = (vps + kWave - 1) / kWave * kWave;
-    if (vps < kWave) vps = kWave;
+    const int64_t quantum = streaming ? 2 * streaming * kWave : kWave;   // whole steps / group pairs
+    vps = (vps + quantum - 1) / quantum * quantum;
+    if (vps < quantum) vps = quantum;
     FwdCfGeom g;
+    g.streaming = streaming;
     g.vecs_per_seg = (int32_t)vps;
     g.n_segs = (int32_t)((max_vecs + vps - 1) / vps);
     const int64_t total = rows * g.n_segs;
