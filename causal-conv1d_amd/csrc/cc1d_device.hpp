@@ -274,6 +274,28 @@ __device__ __forceinline__ void load_weights(const void *weight, const void *bia
         bv[j] = bias == nullptr ? 0.f : ld_weight(bias, w_dtype, c0 + j);
 }
 
+// The same for taps and bias known to be fp32, packed (dim, W) and 16-byte aligned: plain
+// vector loads with no branch on the element type and no use of the loaded values, so a
+// caller can issue further loads before it first touches them.  Without a bias, bv holds
+// unspecified finite-or-not bits that the caller must replace by zero.
+template <int W, int NCH>
+__device__ __forceinline__ void load_weights_f32(const void *weight, const void *bias, int c0,
+                                                 float (&wv)[NCH][W], float (&bv)[NCH]) {
+    constexpr int kAlign = NCH * 4 > 16 ? 16 : NCH * 4;
+    const float *src = static_cast<const float *>(__builtin_assume_aligned(
+        reinterpret_cast<const float *>(weight) + (int64_t)c0 * W, kAlign));
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+        for (int w = 0; w < W; ++w) wv[j][w] = src[j * W + w];
+    // Without a bias the taps are read a second time in its place: the load stays
+    // unconditional and nothing waits for it here.
+    const float *bsrc = bias != nullptr ? reinterpret_cast<const float *>(bias) + c0 : src;
+    bsrc = static_cast<const float *>(__builtin_assume_aligned(bsrc, kAlign));
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) bv[j] = bsrc[j];
+}
+
 // ---------------------------------------------------------------------------------
 // Wave64 lane shifts through DPP (no LDS, no memory).  All 64 lanes must be active.
 //   from_prev_lane: lane i receives lane i-1's value, lane 0 receives `lane0_fill`.

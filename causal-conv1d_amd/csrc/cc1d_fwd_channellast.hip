@@ -72,20 +72,31 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     const int t0 = run * T;                           // < L by construction of n_runs
     const int last = L - 1 - t0;                      // last valid row of this run, run-relative
 
-    float wv[CH][W], bv[CH];
-    load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
-                        g.w_fast != 0, c0, wv, bv);
-    // 16-bit outputs with SiLU: taps and bias carry the factor -log2(e), so the sums below
-    // are already the exponent the activation needs (see silu_from_scaled).
+    // 8-byte lanes exist only for fp32 taps packed (dim, W) (the launcher sees to it): their
+    // loads carry no branch, so everything the run starts with is requested before the first
+    // value is touched.  16-byte lanes take any tap layout and element type.
+    constexpr bool WFAST = CH * E::kBytes == 8;
     constexpr bool SCALED = SILU && !PRECISE;
-    if (SCALED) {
+    float wv[CH][W], bv[CH];
+    if (WFAST) load_weights_f32<W, CH>(p.weight, p.bias, c0, wv, bv);
+    else load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, g.w_fast != 0, c0, wv, bv);
+    // 16-bit outputs with SiLU: taps and bias carry the factor -log2(e), so the sums below
+    // are already the exponent the activation needs (see silu_from_scaled).  Applied by
+    // prepare(), after the first row groups have been requested.
+    auto scale_taps = [&]() {
+        if (WFAST && p.bias == nullptr) {
 #pragma unroll
-        for (int j = 0; j < CH; ++j) {
-            bv[j] *= kSiluPrescale;
-#pragma unroll
-            for (int k = 0; k < W; ++k) wv[j][k] *= kSiluPrescale;
+            for (int j = 0; j < CH; ++j) bv[j] = 0.f;
         }
-    }
+        if (SCALED) {
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                bv[j] *= kSiluPrescale;
+#pragma unroll
+                for (int k = 0; k < W; ++k) wv[j][k] *= kSiluPrescale;
+            }
+        }
+    };
 
     const int64_t xoff = (int64_t)b * p.x_stride_b + c0;
     const int64_t ooff = (int64_t)b * p.out_stride_b + c0;
@@ -96,25 +107,31 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     const uint32_t os = (uint32_t)p.out_stride_l * (uint32_t)sizeof(T_);
     const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
 
-    // Sliding window: xw[i] holds row t-(W-1)+i while row t is being produced.
+    // Sliding window: xw[i] holds row t-(W-1)+i while row t is being produced.  The halo
+    // rows are requested here and unpacked by prepare().
     float xw[W - 1][CH];
     int sqw[W - 1];
+    raw_t halo[W - 1];
 #pragma unroll
     for (int i = 0; i < W - 1; ++i) {
         const int t = t0 - (W - 1) + i;
-        raw_t r = P::zero();
+        halo[i] = P::zero();
         if (t >= 0) {
-            r = *reinterpret_cast<const raw_t *>(xrun - (int64_t)(W - 1 - i) * xs);
+            halo[i] = *reinterpret_cast<const raw_t *>(xrun - (int64_t)(W - 1 - i) * xs);
         } else if (p.initial_states != nullptr) {
-            r = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
-                                       p.init_stride_l, b, c0, t + (W - 1));
+            halo[i] = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
+                                             p.init_stride_l, b, c0, t + (W - 1));
         }
-        P::unpack(r, xw[i]);
         // Rows in front of the sequence hold zeros unless initial_states are given; with
         // zeros a mask changes nothing, so they take the first row's id and do not make
         // the first group look like a boundary.
         sqw[i] = !HAS_SEQ ? 0 : t >= 0 ? seq[i - (W - 1)] : p.initial_states != nullptr ? -1 : seq[-t0];
     }
+    auto prepare = [&]() {
+        scale_taps();
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i) P::unpack(halo[i], xw[i]);
+    };
 
     // CHECKED = false: the whole run lies inside the sequence, so loads and stores are
     // unconditional (the wait counts the compiler derives are then exact and loads stay
@@ -200,6 +217,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
         if (T > 2 * U) {
             load_group(No{}, Yes{}, 0, ra, sa);
             load_group(No{}, Yes{}, U, rb_, sb);
+            prepare();
             compute_group(No{}, 0, ra, sa);
             int i = 2 * U;
             if (T > 4 * U) {
@@ -227,10 +245,12 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
         } else {
             load_group(No{}, Yes{}, 0, ra, sa);
             load_group(No{}, No{}, U, rb_, sb);
+            prepare();
             compute_group(No{}, 0, ra, sa);
             compute_group(No{}, U, rb_, sb);
         }
     } else {
+        prepare();
         for (int i = 0; i <= last; i += U) {
             load_group(Yes{}, No{}, i, ra, sa);
             compute_group(Yes{}, i, ra, sa);
@@ -343,7 +363,9 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
     // 16-byte lane, so twice the waves per SIMD to overlap compute with memory; measured
     // 9% faster at the prefill shape.  fwd_cl_half_vec = -1 selects 16-byte lanes.
     const int full = vec_elems(p.x_dtype);
-    const int ch = tunables().fwd_cl_half_vec < 0 ? full : full / 2;
+    const bool w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width) &&
+                        (p.bias == nullptr || aligned16(p.bias));
+    const int ch = (tunables().fwd_cl_half_vec < 0 || !w_fast) ? full : full / 2;
     FwdClGeom g;
     g.n_colgroups = p.dim / ch;
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
