@@ -9,11 +9,12 @@
 // and one vector store per lane, both fully coalesced along dim, no LDS and no barrier.
 // The only re-read is the (W-1)-row halo in front of each run.
 //
-// Work items (batch, run, vector-column) are laid out flat, so every lane is busy for
-// any dim that is a multiple of CH; lanes of one wave may sit in different runs, which is
-// why seq_idx is tracked per lane.  Workgroups are renumbered so that each of the 8 XCDs
-// (hardware hands workgroups to XCDs round-robin) walks a contiguous slice of that flat
-// order: the run that follows another along seqlen then executes on the same XCD, close
+// A wavefront takes 64 adjacent vector-columns of one (batch, run), so the run's row
+// range and its seq_idx values are scalars; the columns of a row are covered by
+// ceil(dim / (64 CH)) wavefronts, the last one partly idle when dim is not a multiple of
+// 64 CH.  Wavefronts are numbered (batch, run, column block) with the column block
+// fastest, and workgroups are renumbered so that each of the 8 XCDs (hardware hands
+// workgroups to XCDs round-robin) walks a contiguous slice of that order: the run that follows another along seqlen then executes on the same XCD, close
 // in time, and its halo rows are found in that XCD's L2 instead of being fetched from
 // HBM twice.  For the same reason the halo rows and the last rows of a run are accessed
 // with the normal cache policy while everything else streams through (non-temporal).
@@ -25,6 +26,10 @@
 // Rows per register set; two sets are in flight per lane.
 #ifndef CC1D_FWD_CL_UNROLL
 #define CC1D_FWD_CL_UNROLL 8
+#endif
+// The same for 16-byte lanes, whose rows take twice the registers.
+#ifndef CC1D_FWD_CL_UNROLL16
+#define CC1D_FWD_CL_UNROLL16 4
 #endif
 // Workgroups per CU the register budget must allow, for 16- and 8-byte lanes.
 #ifndef CC1D_FWD_CL_OCC16
@@ -43,7 +48,8 @@ struct FwdClGeom {
     int32_t rows_per_run;     // T, a multiple of twice the unroll factor
     int32_t n_runs;           // ceil(seqlen / T)
     int32_t n_colgroups;      // dim / CH
-    uint32_t total;           // batch * n_runs * n_colgroups work items
+    uint32_t waves_per_row;   // ceil(n_colgroups / 64): wavefronts side by side on one row
+    uint32_t total;           // batch * n_runs * waves_per_row wavefronts
     uint32_t blocks_per_xcd;  // grid size / 8
     int32_t w_fast;           // weights_contiguous_f32
     int32_t seq_vec;          // seq_idx rows may be read as 16-byte vectors
@@ -60,10 +66,14 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
 
     // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
     const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
-    const uint32_t gid = block * (uint32_t)kBlock + threadIdx.x;
-    if (gid >= g.total) return;                       // no cross-lane traffic below
-    const uint32_t col = gid % (uint32_t)g.n_colgroups;
-    const uint32_t rb = gid / (uint32_t)g.n_colgroups;
+    // A wavefront never straddles two runs: its batch index, run and row range are scalars,
+    // and so are the sub-sequence ids it reads.
+    const uint32_t wave = block * (uint32_t)(kBlock / kWave) +
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    if (wave >= g.total) return;
+    const uint32_t col = (wave % g.waves_per_row) * (uint32_t)kWave + (threadIdx.x & (kWave - 1));
+    const uint32_t rb = wave / g.waves_per_row;
+    if (col >= (uint32_t)g.n_colgroups) return;       // no cross-lane traffic below
     const int run = (int)(rb % (uint32_t)g.n_runs);
     const int b = (int)(rb / (uint32_t)g.n_runs);
     const int c0 = (int)col * CH;
@@ -129,6 +139,10 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     }
     auto prepare = [&]() {
         scale_taps();
+        if (HAS_SEQ) {
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) sqw[i] = __builtin_amdgcn_readfirstlane(sqw[i]);
+        }
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) P::unpack(halo[i], xw[i]);
     };
@@ -145,7 +159,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
             const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
             const raw_t *src = reinterpret_cast<const raw_t *>(xrun + (uint32_t)i * xs);
             raw[u] = decltype(stream)::value ? __builtin_nontemporal_load(src) : *src;
-            if (HAS_SEQ && (decltype(checked)::value || U % 4 != 0)) sq[u] = seq[i];
+            if (HAS_SEQ && (decltype(checked)::value || U % 4 != 0)) sq[u] = seq[i];   // uniform address
             if (!HAS_SEQ) sq[u] = 0;
         }
         if (HAS_SEQ && !decltype(checked)::value && U % 4 == 0) {
@@ -164,20 +178,25 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     };
 
     // With seq_idx the walk computes every row as if no sub-sequence boundary were near
-    // (no branch in the hot loop) and only records, per lane, the span of row groups whose
+    // (no branch in the hot loop) and only records, per wavefront, the span of row groups whose
     // rows or window are not all of one non-negative id.  Those few rows are redone with
     // masked taps after the walk.
     int redo_lo = T, redo_hi = 0;
     auto compute_group = [&](auto checked, int i0, const raw_t (&raw)[U], const int (&sq)[U]) {
         if (HAS_SEQ) {
-            uint32_t lo = (uint32_t)sq[0], hi = (uint32_t)sq[0];
+            // The ids are the same in every lane: one lane's copy goes to scalar registers
+            // and the bookkeeping runs on the scalar unit.
+            int id[U];
 #pragma unroll
-            for (int u = 1; u < U; ++u) { lo = min(lo, (uint32_t)sq[u]); hi = max(hi, (uint32_t)sq[u]); }
+            for (int u = 0; u < U; ++u) id[u] = __builtin_amdgcn_readfirstlane(sq[u]);
+            uint32_t lo = (uint32_t)id[0], hi = (uint32_t)id[0];
+#pragma unroll
+            for (int u = 1; u < U; ++u) { lo = min(lo, (uint32_t)id[u]); hi = max(hi, (uint32_t)id[u]); }
 #pragma unroll
             for (int k = 0; k < W - 1; ++k) { lo = min(lo, (uint32_t)sqw[k]); hi = max(hi, (uint32_t)sqw[k]); }
             if (lo != hi || (int)hi < 0) { redo_lo = min(redo_lo, i0); redo_hi = max(redo_hi, i0 + U); }
 #pragma unroll
-            for (int k = 0; k < W - 1; ++k) sqw[k] = sq[U - (W - 1) + k];
+            for (int k = 0; k < W - 1; ++k) sqw[k] = id[U - (W - 1) + k];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -274,7 +293,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
                 i = i > last ? last : i;
                 i = before ? 0 : i;
                 P::unpack(*reinterpret_cast<const raw_t *>(xrun + (int64_t)i * xs), xr[q]);
-                const int id = seq[i];
+                const int id = __builtin_amdgcn_readfirstlane(seq[i]);
                 sr[q] = before ? -1 : id;
             }
 #pragma unroll
@@ -318,7 +337,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
 
 template <int DT, int CH, int W, bool HAS_SEQ>
 int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
-    constexpr int U = CC1D_FWD_CL_UNROLL;
+    constexpr int U = CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_UNROLL16 : CC1D_FWD_CL_UNROLL;
     const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
         hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>),
@@ -372,10 +391,11 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
     g.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * elem_bytes(p.x_dtype));
     if (g.rows_per_run == 0) return CC1D_ERR_TOO_LARGE;
     g.n_runs = (p.seqlen + g.rows_per_run - 1) / g.rows_per_run;
-    const int64_t total = (int64_t)p.batch * g.n_runs * g.n_colgroups;
-    if (total >= ((int64_t)1 << 31) - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
+    g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
+    const int64_t total = (int64_t)p.batch * g.n_runs * g.waves_per_row;
+    if (total * kWave >= ((int64_t)1 << 31) - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
     g.total = (uint32_t)total;
-    const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
+    const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
     g.seq_vec = p.seq_idx != nullptr && p.seqlen % 4 == 0 && aligned16(p.seq_idx);
