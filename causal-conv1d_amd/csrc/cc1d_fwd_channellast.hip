@@ -52,12 +52,11 @@ struct FwdClGeom {
     uint32_t total;           // batch * n_runs * waves_per_row wavefronts
     uint32_t blocks_per_xcd;  // grid size / 8
     int32_t w_fast;           // weights_contiguous_f32
-    int32_t seq_vec;          // seq_idx rows may be read as 16-byte vectors
 };
 
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U>
 __global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CC1D_FWD_CL_OCC8))
-fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
+fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t *__restrict__ seq_idx) {
     using E = Elem<DT>;
     using T_ = typename E::type;
     using P = Pack<DT, CH>;
@@ -115,7 +114,9 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     char *orun = reinterpret_cast<char *>(reinterpret_cast<T_ *>(p.out) + ooff + (int64_t)t0 * p.out_stride_l);
     const uint32_t xs = (uint32_t)p.x_stride_l * (uint32_t)sizeof(T_);
     const uint32_t os = (uint32_t)p.out_stride_l * (uint32_t)sizeof(T_);
-    const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+    // seq_idx is a kernel argument of its own, marked as not aliasing anything the kernel
+    // writes: its loads, at wave-uniform addresses, then go through the scalar cache.
+    const int32_t *seq = HAS_SEQ ? seq_idx + (int64_t)b * L + t0 : nullptr;
 
     // Sliding window: xw[i] holds row t-(W-1)+i while row t is being produced.  The halo
     // rows are requested here and unpacked by prepare().
@@ -139,10 +140,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     }
     auto prepare = [&]() {
         scale_taps();
-        if (HAS_SEQ) {
-#pragma unroll
-            for (int i = 0; i < W - 1; ++i) sqw[i] = __builtin_amdgcn_readfirstlane(sqw[i]);
-        }
+
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) P::unpack(halo[i], xw[i]);
     };
@@ -159,21 +157,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
             const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
             const raw_t *src = reinterpret_cast<const raw_t *>(xrun + (uint32_t)i * xs);
             raw[u] = decltype(stream)::value ? __builtin_nontemporal_load(src) : *src;
-            if (HAS_SEQ && (decltype(checked)::value || U % 4 != 0)) sq[u] = seq[i];   // uniform address
-            if (!HAS_SEQ) sq[u] = 0;
-        }
-        if (HAS_SEQ && !decltype(checked)::value && U % 4 == 0) {
-            if (g.seq_vec) {
-#pragma unroll
-                for (int q = 0; q < U / 4; ++q) {
-                    const u32x4 s4 = *reinterpret_cast<const u32x4 *>(seq + i0 + 4 * q);
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) sq[4 * q + k] = (int)s4[k];
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; ++u) sq[u] = seq[i0 + u];
-            }
+            sq[u] = HAS_SEQ ? seq[i] : 0;             // wave-uniform address: a scalar load
         }
     };
 
@@ -184,11 +168,10 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
     int redo_lo = T, redo_hi = 0;
     auto compute_group = [&](auto checked, int i0, const raw_t (&raw)[U], const int (&sq)[U]) {
         if (HAS_SEQ) {
-            // The ids are the same in every lane: one lane's copy goes to scalar registers
-            // and the bookkeeping runs on the scalar unit.
+            // The ids sit in scalar registers and the bookkeeping runs on the scalar unit.
             int id[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) id[u] = __builtin_amdgcn_readfirstlane(sq[u]);
+            for (int u = 0; u < U; ++u) id[u] = sq[u];
             uint32_t lo = (uint32_t)id[0], hi = (uint32_t)id[0];
 #pragma unroll
             for (int u = 1; u < U; ++u) { lo = min(lo, (uint32_t)id[u]); hi = max(hi, (uint32_t)id[u]); }
@@ -293,7 +276,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g) {
                 i = i > last ? last : i;
                 i = before ? 0 : i;
                 P::unpack(*reinterpret_cast<const raw_t *>(xrun + (int64_t)i * xs), xr[q]);
-                const int id = __builtin_amdgcn_readfirstlane(seq[i]);
+                const int id = seq[i];
                 sr[q] = before ? -1 : id;
             }
 #pragma unroll
@@ -341,10 +324,10 @@ int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t st
     const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
         hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>),
-                           dim3(blocks), dim3(kBlock), 0, stream, p, g);
+                           dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx);
     else
         hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>),
-                           dim3(blocks), dim3(kBlock), 0, stream, p, g);
+                           dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx);
     return launch_status();
 }
 
@@ -398,7 +381,6 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
-    g.seq_vec = p.seq_idx != nullptr && p.seqlen % 4 == 0 && aligned16(p.seq_idx);
     const bool half = ch != full;
     switch (p.x_dtype) {
         case CC1D_F32: return half ? launch_width<CC1D_F32, 2>(p, g, stream) : launch_width<CC1D_F32, 4>(p, g, stream);
