@@ -44,14 +44,16 @@ struct BwdClGeom {
     int32_t rows_per_run;     // T, a multiple of twice the unroll factor
     int32_t n_runs;           // ceil(seqlen / T)
     int32_t n_colgroups;      // dim / CH
-    uint32_t total;           // batch * n_runs * n_colgroups work items
+    uint32_t waves_per_row;   // ceil(n_colgroups / 64): wavefronts side by side on one row
+    uint32_t total;           // batch * n_runs * waves_per_row wavefronts
     uint32_t blocks_per_xcd;  // grid size / 8
     int32_t w_fast;           // weights_contiguous_f32
 };
 
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U>
 __global__ void __launch_bounds__(kBlock, CC1D_BWD_CL_OCC)
-bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws) {
+bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws,
+                       const int32_t *__restrict__ seq_idx) {
     using E = Elem<DT>;
     using T_ = typename E::type;
     using P = Pack<DT, CH>;
@@ -60,10 +62,14 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
 
     // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
     const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
-    const uint32_t gid = block * (uint32_t)kBlock + threadIdx.x;
-    if (gid >= g.total) return;                       // no cross-lane traffic below
-    const uint32_t col = gid % (uint32_t)g.n_colgroups;
-    const uint32_t rb = gid / (uint32_t)g.n_colgroups;
+    // A wavefront takes 64 adjacent vector-columns of one (batch, run): its row range and
+    // the sub-sequence ids it reads are scalars.
+    const uint32_t wave = block * (uint32_t)(kBlock / kWave) +
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    if (wave >= g.total) return;
+    const uint32_t col = (wave % g.waves_per_row) * (uint32_t)kWave + (threadIdx.x & (kWave - 1));
+    const uint32_t rb = wave / g.waves_per_row;
+    if (col >= (uint32_t)g.n_colgroups) return;       // no cross-lane traffic below
     const int run = (int)(rb % (uint32_t)g.n_runs);
     const int b = (int)(rb / (uint32_t)g.n_runs);
     const int c0 = (int)col * CH;
@@ -86,70 +92,81 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
     const uint32_t xs = (uint32_t)p.x_stride_l * (uint32_t)sizeof(T_);
     const uint32_t ds = (uint32_t)p.dout_stride_l * (uint32_t)sizeof(T_);
     const uint32_t dxs = (uint32_t)p.dx_stride_l * (uint32_t)sizeof(T_);
-    const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+    // seq_idx is a kernel argument of its own, marked as not aliasing anything the kernel
+    // writes: its loads, at wave-uniform addresses, go through the scalar cache.
+    const int32_t *seq = HAS_SEQ ? seq_idx + (int64_t)b * L + t0 : nullptr;
+
+    using No = std::integral_constant<bool, false>;
+    using Yes = std::integral_constant<bool, true>;
 
     // g[t] = dout[t] * act'(z[t]) from the x window in front of row t; taps that cross a
     // sub-sequence boundary are masked, padding rows (id < 0) have no gradient.
-    auto grad_row = [&](const float (&xwin)[W - 1][CH], const int (&idwin)[W - 1], const float (&xv)[CH],
-                        int cur, float (&gv)[CH]) {
+    // MASKED = false is for rows whose window holds one non-negative id throughout.
+    auto grad_row = [&](auto masked, const float (&xwin)[W - 1][CH], const int (&idwin)[W - 1],
+                        const float (&xv)[CH], int cur, float (&gv)[CH]) __attribute__((always_inline)) {
+        constexpr bool MASKED = HAS_SEQ && decltype(masked)::value;
         if (SILU) {
 #pragma unroll
             for (int j = 0; j < CH; ++j) {
                 float z = bv[j];
 #pragma unroll
                 for (int k = 0; k < W - 1; ++k)
-                    z = fmaf((!HAS_SEQ || idwin[k] == cur) ? xwin[k][j] : 0.f, wv[j][k], z);
+                    z = fmaf((!MASKED || idwin[k] == cur) ? xwin[k][j] : 0.f, wv[j][k], z);
                 z = fmaf(wv[j][W - 1], xv[j], z);
                 gv[j] *= silu_grad<PRECISE>(z);
             }
         }
-        if (HAS_SEQ) {
+        if (MASKED) {
 #pragma unroll
             for (int j = 0; j < CH; ++j) gv[j] = cur < 0 ? 0.f : gv[j];
         }
     };
     // dx[pp] = sum_k weight[W-1-k] * g[pp+k]; gwin holds g[pp .. pp+W-2], gv is g[pp+W-1].
-    auto dx_row = [&](const float (&gwin)[W - 1][CH], const int (&idwin)[W - 1], const float (&gv)[CH],
-                      int cur, float (&dxv)[CH]) {
+    auto dx_row = [&](auto masked, const float (&gwin)[W - 1][CH], const int (&idwin)[W - 1],
+                      const float (&gv)[CH], int cur, float (&dxv)[CH]) __attribute__((always_inline)) {
+        constexpr bool MASKED = HAS_SEQ && decltype(masked)::value;
         const int sp = idwin[0];
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
             float a = wv[j][W - 1] * gwin[0][j];
 #pragma unroll
             for (int k = 1; k < W - 1; ++k)
-                a = fmaf((!HAS_SEQ || idwin[k] == sp) ? gwin[k][j] : 0.f, wv[j][W - 1 - k], a);
-            a = fmaf((!HAS_SEQ || cur == sp) ? gv[j] : 0.f, wv[j][0], a);
+                a = fmaf((!MASKED || idwin[k] == sp) ? gwin[k][j] : 0.f, wv[j][W - 1 - k], a);
+            a = fmaf((!MASKED || cur == sp) ? gv[j] : 0.f, wv[j][0], a);
             dxv[j] = a;
         }
     };
 
     // Windows at row t: xw[k] = x[t-(W-1)+k], gw[k] = g[t-(W-1)+k], sqw[k] the ids.
-    // Filling gw needs the x rows and ids another W-1 steps back.
+    // Filling gw needs the x rows and ids another W-1 steps back.  The rows are requested
+    // here; fill_windows() turns them into the windows once the walk's first row groups have
+    // been requested as well.
     float xw[W - 1][CH], gw[W - 1][CH];
     int sqw[W - 1];
-    {
+    raw_t xh_raw[2 * (W - 1)], dh_raw[W - 1];
+    int sh[2 * (W - 1)];
+#pragma unroll
+    for (int q = 0; q < 2 * (W - 1); ++q) {
+        const int t = t0 - 2 * (W - 1) + q;
+        xh_raw[q] = P::zero();
+        if (t >= 0) {
+            xh_raw[q] = *reinterpret_cast<const raw_t *>(xrun - (int64_t)(2 * (W - 1) - q) * xs);
+        } else if (p.initial_states != nullptr && t >= -(W - 1)) {
+            xh_raw[q] = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
+                                               p.init_stride_l, b, c0, t + (W - 1));
+        }
+        sh[q] = (HAS_SEQ && t >= 0) ? seq[q - 2 * (W - 1)] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < W - 1; ++k) {
+        const int t = t0 - (W - 1) + k;
+        dh_raw[k] = P::zero();
+        if (t >= 0) dh_raw[k] = *reinterpret_cast<const raw_t *>(drun - (int64_t)(W - 1 - k) * ds);
+    }
+    auto fill_windows = [&]() __attribute__((always_inline)) {
         float xh[2 * (W - 1)][CH];
-        int sh[2 * (W - 1)];
-        raw_t dh[W - 1];
 #pragma unroll
-        for (int q = 0; q < 2 * (W - 1); ++q) {
-            const int t = t0 - 2 * (W - 1) + q;
-            raw_t r = P::zero();
-            if (t >= 0) {
-                r = *reinterpret_cast<const raw_t *>(xrun - (int64_t)(2 * (W - 1) - q) * xs);
-            } else if (p.initial_states != nullptr && t >= -(W - 1)) {
-                r = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
-                                           p.init_stride_l, b, c0, t + (W - 1));
-            }
-            P::unpack(r, xh[q]);
-            sh[q] = (HAS_SEQ && t >= 0) ? seq[q - 2 * (W - 1)] : -1;
-        }
-#pragma unroll
-        for (int k = 0; k < W - 1; ++k) {
-            const int t = t0 - (W - 1) + k;
-            dh[k] = P::zero();
-            if (t >= 0) dh[k] = *reinterpret_cast<const raw_t *>(drun - (int64_t)(W - 1 - k) * ds);
-        }
+        for (int q = 0; q < 2 * (W - 1); ++q) P::unpack(xh_raw[q], xh[q]);
 #pragma unroll
         for (int k = 0; k < W - 1; ++k) {
             float xwin[W - 1][CH];
@@ -160,12 +177,42 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
 #pragma unroll
                 for (int j = 0; j < CH; ++j) xwin[i][j] = xh[k + i][j];
             }
-            P::unpack(dh[k], gw[k]);                  // zero in front of the sequence
-            grad_row(xwin, idwin, xh[k + W - 1], sh[k + W - 1], gw[k]);
+            P::unpack(dh_raw[k], gw[k]);              // zero in front of the sequence
+            grad_row(Yes{}, xwin, idwin, xh[k + W - 1], sh[k + W - 1], gw[k]);
 #pragma unroll
             for (int j = 0; j < CH; ++j) xw[k][j] = xh[k + W - 1][j];
             sqw[k] = sh[k + W - 1];
         }
+    };
+
+    // With seq_idx, a run whose rows and halo all carry one non-negative id needs no masks
+    // at all; the ids are scalars, so finding that out costs the vector unit nothing, and the
+    // run then takes the same arithmetic as a run without seq_idx.
+    bool mixed = false;
+    if (HAS_SEQ) {
+        const int i_lo = t0 >= 2 * (W - 1) ? -2 * (W - 1) : -t0;
+        uint32_t lo = (uint32_t)seq[i_lo], hi = lo;
+        // Consecutive ids arrive through wide scalar loads; 64 at a time so that the loads
+        // of a trip overlap, and the ragged end re-reads the last 16.
+        auto scan = [&](auto n, int i) __attribute__((always_inline)) {
+#pragma unroll
+            for (int k = 0; k < decltype(n)::value; ++k) {
+                const uint32_t v = (uint32_t)seq[i + k];
+                lo = min(lo, v);
+                hi = max(hi, v);
+            }
+        };
+        int i = i_lo;
+        for (; i + 63 <= last; i += 64) scan(std::integral_constant<int, 64>{}, i);
+        for (; i + 15 <= last; i += 16) scan(std::integral_constant<int, 16>{}, i);
+        if (i <= last) {
+            if (last - 15 >= i_lo) {
+                scan(std::integral_constant<int, 16>{}, last - 15);
+            } else {
+                for (; i <= last; ++i) scan(std::integral_constant<int, 1>{}, i);
+            }
+        }
+        mixed = lo != hi || (int)hi < 0;
     }
 
     float dW[CH][W], dB[CH];
@@ -182,7 +229,7 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
     // ragged or short runs (rows past the end re-read the last valid row and are inert).
     // STREAM: non-temporal loads; the last rows of a run are read with the normal policy
     // because the following run needs them again as its halo.
-    auto load_group = [&](auto checked, auto stream, int i0, raw_t (&rx)[U], raw_t (&rd)[U], int (&sq)[U]) {
+    auto load_group = [&](auto checked, auto stream, int i0, raw_t (&rx)[U], raw_t (&rd)[U], int (&sq)[U]) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
@@ -193,7 +240,9 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
             sq[u] = HAS_SEQ ? seq[i] : 0;
         }
     };
-    auto compute_group = [&](auto checked, int i0, const raw_t (&rx)[U], const raw_t (&rd)[U], const int (&sq)[U]) {
+    auto compute_group = [&](auto checked, auto masked, int i0, const raw_t (&rx)[U], const raw_t (&rd)[U],
+                            const int (&sq)[U]) __attribute__((always_inline)) {
+        constexpr bool MASKED = HAS_SEQ && decltype(masked)::value;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (decltype(checked)::value && i0 + u > last) continue;   // past the end: inert
@@ -201,16 +250,16 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
             float xv[CH], gv[CH], dxv[CH];
             P::unpack(rx[u], xv);
             P::unpack(rd[u], gv);
-            grad_row(xw, sqw, xv, cur, gv);
+            grad_row(masked, xw, sqw, xv, cur, gv);
 #pragma unroll
             for (int j = 0; j < CH; ++j) {
                 dB[j] += gv[j];
 #pragma unroll
                 for (int k = 0; k < W - 1; ++k)
-                    dW[j][k] = fmaf(gv[j], (!HAS_SEQ || sqw[k] == cur) ? xw[k][j] : 0.f, dW[j][k]);
+                    dW[j][k] = fmaf(gv[j], (!MASKED || sqw[k] == cur) ? xw[k][j] : 0.f, dW[j][k]);
                 dW[j][W - 1] = fmaf(gv[j], xv[j], dW[j][W - 1]);
             }
-            dx_row(gw, sqw, gv, cur, dxv);
+            dx_row(masked, gw, sqw, gv, cur, dxv);
             if (!decltype(checked)::value) {
                 __builtin_nontemporal_store(P::pack(dxv), reinterpret_cast<raw_t *>(dxrun + (uint32_t)(i0 + u) * dxs));
             } else {
@@ -234,47 +283,50 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
             sqw[W - 2] = cur;
         }
     };
-
-    using No = std::integral_constant<bool, false>;
-    using Yes = std::integral_constant<bool, true>;
     // Run 0 routes positions in front of the sequence through the checked form of its first
     // group only, so that group must hold all W-1 of them.
     static_assert(U >= W - 1, "the first group must cover the window");
     raw_t xa[U], da[U], xb[U], db[U];
     int sa[U], sb[U];
-    if (full && T >= 6 * U) {
-        // Two register sets in ping-pong: while one group of U rows is computed and stored,
-        // the loads of the next two groups are in flight, and nothing is copied at the loop
-        // edge.  The first and the last pair of groups are peeled, so the loop is entered
-        // in exactly the state its back edge leaves and the wait counts stay exact.
-        load_group(No{}, Yes{}, 0, xa, da, sa);
-        load_group(No{}, Yes{}, U, xb, db, sb);
-        if (run > 0) compute_group(No{}, 0, xa, da, sa);
-        else compute_group(Yes{}, 0, xa, da, sa);     // rows in front of the sequence: dinitial_states
-        load_group(No{}, Yes{}, 2 * U, xa, da, sa);
-        compute_group(No{}, U, xb, db, sb);
-        load_group(No{}, Yes{}, 3 * U, xb, db, sb);
-        int i = 2 * U;
+    auto walk = [&](auto masked) __attribute__((always_inline)) {
+        if (full && T >= 6 * U) {
+            // Two register sets in ping-pong: while one group of U rows is computed and stored,
+            // the loads of the next two groups are in flight, and nothing is copied at the loop
+            // edge.  The first and the last pair of groups are peeled, so the loop is entered
+            // in exactly the state its back edge leaves and the wait counts stay exact.
+            load_group(No{}, Yes{}, 0, xa, da, sa);
+            load_group(No{}, Yes{}, U, xb, db, sb);
+            fill_windows();
+            if (run > 0) compute_group(No{}, masked, 0, xa, da, sa);
+            else compute_group(Yes{}, masked, 0, xa, da, sa);   // positions in front of the sequence
+            load_group(No{}, Yes{}, 2 * U, xa, da, sa);
+            compute_group(No{}, masked, U, xb, db, sb);
+            load_group(No{}, Yes{}, 3 * U, xb, db, sb);
+            int i = 2 * U;
 #pragma clang loop unroll(disable)
-        for (; i + 4 * U < T; i += 2 * U) {
-            compute_group(No{}, i, xa, da, sa);
-            load_group(No{}, Yes{}, i + 2 * U, xa, da, sa);
-            compute_group(No{}, i + U, xb, db, sb);
-            load_group(No{}, Yes{}, i + 3 * U, xb, db, sb);
+            for (; i + 4 * U < T; i += 2 * U) {
+                compute_group(No{}, masked, i, xa, da, sa);
+                load_group(No{}, Yes{}, i + 2 * U, xa, da, sa);
+                compute_group(No{}, masked, i + U, xb, db, sb);
+                load_group(No{}, Yes{}, i + 3 * U, xb, db, sb);
+            }
+            // i + 4U == T: the run's last 2U rows stay cached for the next run's halo.
+            compute_group(No{}, masked, i, xa, da, sa);
+            load_group(No{}, No{}, i + 2 * U, xa, da, sa);
+            compute_group(No{}, masked, i + U, xb, db, sb);
+            load_group(No{}, No{}, i + 3 * U, xb, db, sb);
+            compute_group(No{}, masked, i + 2 * U, xa, da, sa);
+            compute_group(No{}, masked, i + 3 * U, xb, db, sb);
+        } else {
+            fill_windows();
+            for (int i = 0; i <= last; i += U) {
+                load_group(Yes{}, No{}, i, xa, da, sa);
+                compute_group(Yes{}, masked, i, xa, da, sa);
+            }
         }
-        // i + 4U == T: the run's last 2U rows stay cached for the next run's halo.
-        compute_group(No{}, i, xa, da, sa);
-        load_group(No{}, No{}, i + 2 * U, xa, da, sa);
-        compute_group(No{}, i + U, xb, db, sb);
-        load_group(No{}, No{}, i + 3 * U, xb, db, sb);
-        compute_group(No{}, i + 2 * U, xa, da, sa);
-        compute_group(No{}, i + 3 * U, xb, db, sb);
-    } else {
-        for (int i = 0; i <= last; i += U) {
-            load_group(Yes{}, No{}, i, xa, da, sa);
-            compute_group(Yes{}, i, xa, da, sa);
-        }
-    }
+    };
+    if (HAS_SEQ && mixed) walk(Yes{});
+    else walk(No{});
 
     // The sequence's last run closes it: dx[L-(W-1) .. L) see no further g (zero past the
     // end) and take dfinal_states; with seqlen < W-1 part of that lands in dinitial_states
@@ -287,7 +339,7 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
         for (int k = 0; k < W - 1; ++k) {
             const int pp = L - (W - 1) + k;
             float dxv[CH];
-            dx_row(gw, sqw, zero, -1, dxv);
+            dx_row(Yes{}, gw, sqw, zero, -1, dxv);
             if (p.dfinal_states != nullptr) {
                 const raw_t fr = load_state_row<DT, CH>(p.dfinal_states, p.dfinal_stride_b, p.dfinal_stride_c,
                                                         p.dfinal_stride_l, b, c0, k);
@@ -410,10 +462,11 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     if ((int64_t)(T + U2) * row_bytes >= ((int64_t)1 << 31)) return false;
     g.rows_per_run = T;
     g.n_runs = (p.seqlen + T - 1) / T;
-    const int64_t total = (int64_t)p.batch * g.n_runs * g.n_colgroups;
-    if (total >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
+    g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
+    const int64_t total = (int64_t)p.batch * g.n_runs * g.waves_per_row;
+    if (total * kWave >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
     g.total = (uint32_t)total;
-    const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
+    const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
     return true;
@@ -424,9 +477,9 @@ int launch_instance(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hip
     constexpr int U = CC1D_BWD_CL_UNROLL;
     const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws);
+        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
     else
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws);
+        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
     return launch_status();
 }
 
