@@ -86,10 +86,9 @@ def causal_conv1d_fwd_function(
 ) -> torch.Tensor:
     """out = empty_like(x), filled by the forward kernel (cpp_functions.py:94-114)."""
     out = torch.empty_like(x)
-    _causal_conv1d_fwd_cpp(
-        x=x, weight=weight, bias=bias, seq_idx=seq_idx, initial_states=initial_states,
-        out=out, final_states_out=final_states_out, silu_activation=silu_activation,
-    )
+    # Positional on purpose: torch.compile rejects a keyword argument named `out` that is
+    # not contiguous, which a channel-last output never is.
+    _causal_conv1d_fwd_cpp(x, weight, bias, seq_idx, initial_states, out, final_states_out, silu_activation)
     return out
 
 
@@ -119,11 +118,8 @@ def causal_conv1d_bwd_function(
         dinitial_states = torch.empty(
             batch, width - 1, dim, device=x.device, dtype=x.dtype
         ).transpose(1, 2)
-    _causal_conv1d_bwd_cpp(
-        x=x, weight=weight, bias=bias, dout=dout, seq_idx=seq_idx,
-        initial_states=initial_states, dfinal_states=dfinal_states, dx=dx, dweight=dweight,
-        dbias=dbias, dinitial_states=dinitial_states, silu_activation=silu_activation,
-    )
+    _causal_conv1d_bwd_cpp(x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
+                           dx, dweight, dbias, dinitial_states, silu_activation)
     dweight = dweight.type_as(weight)
     if dbias is not None:
         dbias = dbias.type_as(bias)
@@ -141,9 +137,5 @@ def causal_conv1d_update_function(
 ) -> torch.Tensor:
     """out = empty_like(x); conv_state is advanced in place (cpp_functions.py:163-183)."""
     out = torch.empty_like(x)
-    _causal_conv1d_update_cpp(
-        x=x, conv_state=conv_state, weight=weight, bias=bias, out=out,
-        silu_activation=silu_activation, cache_seqlens=cache_seqlens,
-        conv_state_indices=conv_state_indices,
-    )
+    _causal_conv1d_update_cpp(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices)
     return out
