@@ -1,0 +1,142 @@
+#!/usr/bin/env python
+"""Times one operator of the package at a shape given on the command line and prints
+microseconds per call, achieved GB/s against the bytes the operator must move, and peak
+device memory.  The role of tests/benchmark_determinism_kernels.py in the reference, for
+all four operators; there is no deterministic/non-deterministic pair to compare because the
+backward here is always a fixed-order two-stage sum.
+
+  python benchmark_ops.py --op fwd --batch 8 --dim 5376 --seqlen 2048 --channel-last --seq-idx
+  python benchmark_ops.py --op bwd --batch 4 --dim 4096 --seqlen 8192 --dtype fp16 --states
+  python benchmark_ops.py --op update --batch 256 --dim 5376 --state-len 8 --circular
+  python benchmark_ops.py --op varlen --batch 64 --dim 5376 --seqlen 1024
+"""
+import argparse
+import gc
+import os
+import statistics
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+import torch
+
+from causal_conv1d import causal_conv1d_fn, causal_conv1d_update, causal_conv1d_varlen_states
+from causal_conv1d.cpp_functions import causal_conv1d_bwd_function
+
+HBM_PEAK_GBS = 8000.0
+
+
+def timed(fn, warmup, rep, iters):
+    """Median over `iters` groups of `rep` back-to-back calls, in microseconds per call."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    groups = []
+    for _ in range(iters):
+        start.record()
+        for _ in range(rep):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        groups.append(start.elapsed_time(end) * 1e3 / rep)
+    return statistics.median(groups)
+
+
+def peak_mb(fn):
+    fn()
+    torch.cuda.synchronize()
+    gc.collect()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    fn()
+    torch.cuda.synchronize()
+    return (torch.cuda.max_memory_allocated() - base) / 2**20
+
+
+def nbytes(*ts):
+    return sum(t.numel() * t.element_size() for t in ts if t is not None)
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--op", choices=["fwd", "bwd", "update", "varlen"], default="fwd")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dim", type=int, default=5376)
+    ap.add_argument("--seqlen", type=int, default=2048, help="per-sequence length (varlen: mean length)")
+    ap.add_argument("--width", type=int, default=4, choices=[2, 3, 4])
+    ap.add_argument("--dtype", choices=["fp16", "bf16", "fp32"], default="bf16")
+    ap.add_argument("--channel-last", action="store_true")
+    ap.add_argument("--seq-idx", action="store_true", help="fwd/bwd: 4 packed sub-sequences per row")
+    ap.add_argument("--states", action="store_true", help="fwd/bwd: initial_states and final states")
+    ap.add_argument("--no-bias", action="store_true")
+    ap.add_argument("--activation", choices=["none", "silu"], default="silu")
+    ap.add_argument("--state-len", type=int, default=3, help="update/varlen: conv_state length")
+    ap.add_argument("--circular", action="store_true", help="update: cache_seqlens ring buffer")
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--rep", type=int, default=50)
+    ap.add_argument("--iters", type=int, default=20)
+    a = ap.parse_args()
+
+    dev = "cuda"
+    dtype = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[a.dtype]
+    act = None if a.activation == "none" else "silu"
+    B, D, L, W = a.batch, a.dim, a.seqlen, a.width
+    weight = torch.rand(D, W, device=dev) - 0.5
+    bias = None if a.no_bias else torch.rand(D, device=dev) - 0.5
+
+    def make(shape_bld):
+        b, d, l = shape_bld
+        if a.channel_last:
+            return torch.randn(b, l, d, device=dev, dtype=dtype).transpose(1, 2)
+        return torch.randn(b, d, l, device=dev, dtype=dtype)
+
+    if a.op in ("fwd", "bwd"):
+        x = make((B, D, L))
+        seq = None
+        if a.seq_idx:
+            seq = (torch.arange(L, device=dev, dtype=torch.int32) * 4 // L).expand(B, L).contiguous()
+        init = torch.randn(B, W - 1, D, device=dev, dtype=dtype).transpose(1, 2) if a.states else None
+        if a.op == "fwd":
+            fn = lambda: causal_conv1d_fn(x, weight, bias, seq_idx=seq, initial_states=init,
+                                          return_final_states=a.states, activation=act)
+            moved = 2 * nbytes(x) + nbytes(seq, weight, bias, init) + (nbytes(init) if a.states else 0)
+        else:
+            dout = torch.randn_like(x)
+            dx = torch.empty_like(x)
+            dfin = torch.randn(B, W - 1, D, device=dev, dtype=dtype).transpose(1, 2) if a.states else None
+            fn = lambda: causal_conv1d_bwd_function(x, weight, bias, dout, seq, init, dfin, dx, a.states, act == "silu")
+            moved = 3 * nbytes(x) + nbytes(seq, weight, bias, init, dfin) + (nbytes(init) if a.states else 0) + \
+                (W + (0 if a.no_bias else 1)) * D * 4
+    elif a.op == "update":
+        S = a.state_len
+        x = torch.randn(B, D, device=dev, dtype=dtype)
+        state = torch.randn(B, S, D, device=dev, dtype=dtype).transpose(1, 2)
+        cache = torch.randint(0, 1000, (B,), device=dev, dtype=torch.int32) if a.circular else None
+        fn = lambda: causal_conv1d_update(x, state, weight, bias, activation=act, cache_seqlens=cache)
+        per_chan = (1 + (W - 1) + 1 + 1) if a.circular else (1 + S + S + 1)   # x, state reads, state writes, out
+        moved = per_chan * B * D * x.element_size() + nbytes(weight, bias, cache)
+    else:
+        S = a.state_len
+        lens = torch.randint(max(1, L // 2), L + L // 2, (B,))
+        cu = torch.zeros(B + 1, dtype=torch.int32)
+        cu[1:] = lens.cumsum(0)
+        x = torch.randn(int(cu[-1]), D, device=dev, dtype=dtype)
+        cu = cu.to(dev)
+        fn = lambda: causal_conv1d_varlen_states(x, cu, S)
+        moved = 2 * B * D * S * x.element_size() + nbytes(cu)
+
+    with torch.no_grad():
+        us = timed(fn, a.warmup, a.rep, a.iters)
+        mb = peak_mb(fn)
+    gbs = moved / us / 1e3
+    print("GPU: %s" % torch.cuda.get_device_name(0))
+    print("op=%s batch=%d dim=%d seqlen=%d width=%d dtype=%s channel_last=%s seq_idx=%s states=%s bias=%s act=%s"
+          % (a.op, B, D, L, W, a.dtype, a.channel_last, a.seq_idx, a.states, not a.no_bias, a.activation))
+    print("%10s %12s %10s %12s %10s" % ("us/call", "bytes moved", "GB/s", "% of 8 TB/s", "peak MB"))
+    print("%10.2f %12d %10.1f %12.1f %10.1f" % (us, moved, gbs, 100 * gbs / HBM_PEAK_GBS, mb))
+
+
+if __name__ == "__main__":
+    main()
