@@ -1,141 +1,85 @@
-"""torch.library registration of the three mutating device ops and the allocating
-wrappers around them.  Same op names, argument order and ownership rules as
-causal_conv1d/cpp_functions.py:11-183 of the reference: Python allocates every output,
-the extension only writes into them.
+"""The three device operators as torch.library custom ops, and the allocating wrappers the
+autograd layer calls.
 
-The extension module `causal_conv1d_cuda` is required: importing this file without it
-raises ImportError (there is no fallback path).
+Op names, argument order and ownership follow causal_conv1d/cpp_functions.py:11-183 of the
+reference, because downstream code reaches the kernels through exactly these names
+(torch.ops.DaoAILab._causal_conv1d_{fwd,bwd,update}_cpp): Python owns every output tensor, the
+extension only writes into what it is given.  There is no fallback: without the compiled
+module `causal_conv1d_cuda` this file does not import.
 """
 from typing import Optional, Tuple
 
 import torch
+from torch import Tensor
 
-import causal_conv1d_cuda
+import causal_conv1d_cuda as _ext
 
 LIBRARY_NAME = "DaoAILab"
+_Opt = Optional[Tensor]
 
 
-@torch.library.custom_op(
-    f"{LIBRARY_NAME}::_causal_conv1d_fwd_cpp", mutates_args={"out", "final_states_out"}
-)
-def _causal_conv1d_fwd_cpp(
-    x: torch.Tensor,
-    weight: torch.Tensor,
-    bias: Optional[torch.Tensor],
-    seq_idx: Optional[torch.Tensor],
-    initial_states: Optional[torch.Tensor],
-    out: torch.Tensor,
-    final_states_out: Optional[torch.Tensor],
-    silu_activation: bool,
-) -> None:
-    causal_conv1d_cuda.causal_conv1d_fwd(
-        x, weight, bias, seq_idx, initial_states, out, final_states_out, silu_activation
-    )
+def _device_op(name, mutated):
+    """Registers `fn` as DaoAILab::<name>, declaring which arguments it writes."""
+    return torch.library.custom_op("%s::%s" % (LIBRARY_NAME, name), mutates_args=set(mutated))
 
 
-@torch.library.custom_op(
-    f"{LIBRARY_NAME}::_causal_conv1d_bwd_cpp",
-    mutates_args={"dfinal_states", "dx", "dweight", "dbias", "dinitial_states"},
-)
-def _causal_conv1d_bwd_cpp(
-    x: torch.Tensor,
-    weight: torch.Tensor,
-    bias: Optional[torch.Tensor],
-    dout: torch.Tensor,
-    seq_idx: Optional[torch.Tensor],
-    initial_states: Optional[torch.Tensor],
-    dfinal_states: Optional[torch.Tensor],
-    dx: torch.Tensor,
-    dweight: torch.Tensor,
-    dbias: Optional[torch.Tensor],
-    dinitial_states: Optional[torch.Tensor],
-    silu_activation: bool,
-) -> None:
-    causal_conv1d_cuda.causal_conv1d_bwd(
-        x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
-        dx, dweight, dbias, dinitial_states, silu_activation,
-    )
+@_device_op("_causal_conv1d_fwd_cpp", ("out", "final_states_out"))
+def _causal_conv1d_fwd_cpp(x: Tensor, weight: Tensor, bias: _Opt, seq_idx: _Opt, initial_states: _Opt,
+                           out: Tensor, final_states_out: _Opt, silu_activation: bool) -> None:
+    _ext.causal_conv1d_fwd(x, weight, bias, seq_idx, initial_states, out, final_states_out, silu_activation)
 
 
-@torch.library.custom_op(
-    f"{LIBRARY_NAME}::_causal_conv1d_update_cpp", mutates_args={"out", "conv_state"}
-)
-def _causal_conv1d_update_cpp(
-    x: torch.Tensor,
-    conv_state: torch.Tensor,
-    weight: torch.Tensor,
-    bias: Optional[torch.Tensor],
-    out: torch.Tensor,
-    silu_activation: bool,
-    cache_seqlens: Optional[torch.Tensor],
-    conv_state_indices: Optional[torch.Tensor],
-) -> None:
-    causal_conv1d_cuda.causal_conv1d_update(
-        x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices
-    )
+@_device_op("_causal_conv1d_bwd_cpp", ("dfinal_states", "dx", "dweight", "dbias", "dinitial_states"))
+def _causal_conv1d_bwd_cpp(x: Tensor, weight: Tensor, bias: _Opt, dout: Tensor, seq_idx: _Opt,
+                           initial_states: _Opt, dfinal_states: _Opt, dx: Tensor, dweight: Tensor,
+                           dbias: _Opt, dinitial_states: _Opt, silu_activation: bool) -> None:
+    _ext.causal_conv1d_bwd(x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
+                           dx, dweight, dbias, dinitial_states, silu_activation)
 
 
-def causal_conv1d_fwd_function(
-    x: torch.Tensor,
-    weight: torch.Tensor,
-    bias: Optional[torch.Tensor],
-    seq_idx: Optional[torch.Tensor],
-    initial_states: Optional[torch.Tensor],
-    final_states_out: Optional[torch.Tensor],
-    silu_activation: bool,
-) -> torch.Tensor:
-    """out = empty_like(x), filled by the forward kernel (cpp_functions.py:94-114)."""
+@_device_op("_causal_conv1d_update_cpp", ("out", "conv_state"))
+def _causal_conv1d_update_cpp(x: Tensor, conv_state: Tensor, weight: Tensor, bias: _Opt, out: Tensor,
+                              silu_activation: bool, cache_seqlens: _Opt, conv_state_indices: _Opt) -> None:
+    _ext.causal_conv1d_update(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices)
+
+
+def _states_like(x: Tensor, width: int) -> Tensor:
+    """A (batch, dim, width-1) tensor with unit stride along dim, the layout the kernels
+    write states in fastest."""
+    batch, dim = x.shape[0], x.shape[1]
+    return torch.empty(batch, width - 1, dim, device=x.device, dtype=x.dtype).transpose(1, 2)
+
+
+# The ops below are called positionally on purpose: torch.compile rejects a keyword argument
+# named `out` that is not contiguous, which a channel-last output never is.
+
+def causal_conv1d_fwd_function(x: Tensor, weight: Tensor, bias: _Opt, seq_idx: _Opt, initial_states: _Opt,
+                               final_states_out: _Opt, silu_activation: bool) -> Tensor:
+    """Allocates `out` in x's layout and fills it; `final_states_out`, if given, is filled too."""
     out = torch.empty_like(x)
-    # Positional on purpose: torch.compile rejects a keyword argument named `out` that is
-    # not contiguous, which a channel-last output never is.
     _causal_conv1d_fwd_cpp(x, weight, bias, seq_idx, initial_states, out, final_states_out, silu_activation)
     return out
 
 
-def causal_conv1d_bwd_function(
-    x: torch.Tensor,
-    weight: torch.Tensor,
-    bias: Optional[torch.Tensor],
-    dout: torch.Tensor,
-    seq_idx: Optional[torch.Tensor],
-    initial_states: Optional[torch.Tensor],
-    dfinal_states: Optional[torch.Tensor],
-    dx: Optional[torch.Tensor],
-    return_dinitial_states: bool,
-    silu_activation: bool,
-) -> Tuple[Optional[torch.Tensor], ...]:
-    """Allocates dx (unless given), fp32 zeroed dweight/dbias and a channel-last
-    dinitial_states, runs the backward kernels and casts dweight/dbias to the
-    parameter dtype (cpp_functions.py:117-160)."""
-    batch, dim = x.shape[:2]
-    width = weight.shape[-1]
-    if dx is None:
-        dx = torch.empty_like(x)
-    dweight = torch.zeros_like(weight, dtype=torch.float32)
-    dbias = torch.zeros_like(bias, dtype=torch.float32) if bias is not None else None
-    dinitial_states = None
-    if return_dinitial_states:
-        dinitial_states = torch.empty(
-            batch, width - 1, dim, device=x.device, dtype=x.dtype
-        ).transpose(1, 2)
+def causal_conv1d_bwd_function(x: Tensor, weight: Tensor, bias: _Opt, dout: Tensor, seq_idx: _Opt,
+                               initial_states: _Opt, dfinal_states: _Opt, dx: _Opt,
+                               return_dinitial_states: bool, silu_activation: bool) -> Tuple[_Opt, ...]:
+    """Returns (dx, dweight, dbias, dinitial_states).  dx may be supplied by the caller; dweight
+    and dbias are accumulated in fp32 buffers that start at zero (the kernels add into them)
+    and come back in the parameters' dtype."""
+    dx = torch.empty_like(x) if dx is None else dx
+    dweight32 = torch.zeros_like(weight, dtype=torch.float32)
+    dbias32 = None if bias is None else torch.zeros_like(bias, dtype=torch.float32)
+    dinitial_states = _states_like(x, weight.shape[-1]) if return_dinitial_states else None
     _causal_conv1d_bwd_cpp(x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
-                           dx, dweight, dbias, dinitial_states, silu_activation)
-    dweight = dweight.type_as(weight)
-    if dbias is not None:
-        dbias = dbias.type_as(bias)
-    return dx, dweight, dbias, dinitial_states
+                           dx, dweight32, dbias32, dinitial_states, silu_activation)
+    dbias = None if dbias32 is None else dbias32.type_as(bias)
+    return dx, dweight32.type_as(weight), dbias, dinitial_states
 
 
-def causal_conv1d_update_function(
-    x: torch.Tensor,
-    conv_state: torch.Tensor,
-    weight: torch.Tensor,
-    bias: Optional[torch.Tensor],
-    silu_activation: bool,
-    cache_seqlens: Optional[torch.Tensor],
-    conv_state_indices: Optional[torch.Tensor],
-) -> torch.Tensor:
-    """out = empty_like(x); conv_state is advanced in place (cpp_functions.py:163-183)."""
+def causal_conv1d_update_function(x: Tensor, conv_state: Tensor, weight: Tensor, bias: _Opt,
+                                  silu_activation: bool, cache_seqlens: _Opt, conv_state_indices: _Opt) -> Tensor:
+    """Allocates `out` like x; conv_state is advanced in place."""
     out = torch.empty_like(x)
     _causal_conv1d_update_cpp(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices)
     return out
