@@ -444,9 +444,10 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     int T = tunables().bwd_cl_rows;
     // Runs of 128 rows: the halo in front of a run and its partial-sum planes then cost about
     // 5% of the tensor traffic while the prefill shape still launches 2688 wavefronts; measured
-    // best against 32, 64 and 256 there.
+    // best against 32, 64 and 256 there.  With seq_idx 64 rows do better: fewer runs then
+    // contain a sub-sequence boundary and need the masked walk.
     if (T <= 0) {
-        T = 128;
+        T = p.seq_idx != nullptr ? 64 : 128;
         // Small problems: shorter runs until about 8 wavefronts per CU exist.
         const int64_t target_lanes = (int64_t)256 * 8 * kWave;
         while (T > 32 && (int64_t)p.batch * g.n_colgroups * ((p.seqlen + T - 1) / T) < target_lanes) T >>= 1;
