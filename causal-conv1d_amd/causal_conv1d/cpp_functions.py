@@ -1,5 +1,5 @@
-"""The three device operators as torch.library custom ops, and the allocating wrappers the
-autograd layer calls.
+"""The three device operators as torch.library ops, and the allocating wrappers the autograd
+layer calls.
 
 Op names, argument order and ownership follow causal_conv1d/cpp_functions.py:11-183 of the
 reference, because downstream code reaches the kernels through exactly these names
@@ -12,35 +12,16 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor
 
-import causal_conv1d_cuda as _ext
+import causal_conv1d_cuda as _ext  # noqa: F401  (loading it registers the DaoAILab ops with the dispatcher)
 
 LIBRARY_NAME = "DaoAILab"
 _Opt = Optional[Tensor]
 
-
-def _device_op(name, mutated):
-    """Registers `fn` as DaoAILab::<name>, declaring which arguments it writes."""
-    return torch.library.custom_op("%s::%s" % (LIBRARY_NAME, name), mutates_args=set(mutated))
-
-
-@_device_op("_causal_conv1d_fwd_cpp", ("out", "final_states_out"))
-def _causal_conv1d_fwd_cpp(x: Tensor, weight: Tensor, bias: _Opt, seq_idx: _Opt, initial_states: _Opt,
-                           out: Tensor, final_states_out: _Opt, silu_activation: bool) -> None:
-    _ext.causal_conv1d_fwd(x, weight, bias, seq_idx, initial_states, out, final_states_out, silu_activation)
-
-
-@_device_op("_causal_conv1d_bwd_cpp", ("dfinal_states", "dx", "dweight", "dbias", "dinitial_states"))
-def _causal_conv1d_bwd_cpp(x: Tensor, weight: Tensor, bias: _Opt, dout: Tensor, seq_idx: _Opt,
-                           initial_states: _Opt, dfinal_states: _Opt, dx: Tensor, dweight: Tensor,
-                           dbias: _Opt, dinitial_states: _Opt, silu_activation: bool) -> None:
-    _ext.causal_conv1d_bwd(x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
-                           dx, dweight, dbias, dinitial_states, silu_activation)
-
-
-@_device_op("_causal_conv1d_update_cpp", ("out", "conv_state"))
-def _causal_conv1d_update_cpp(x: Tensor, conv_state: Tensor, weight: Tensor, bias: _Opt, out: Tensor,
-                              silu_activation: bool, cache_seqlens: _Opt, conv_state_indices: _Opt) -> None:
-    _ext.causal_conv1d_update(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices)
+# The ops are defined in C++ inside the extension (schema with the written arguments marked,
+# a no-op meta kernel for tracing), so a call costs a dispatcher hop and no Python trampoline.
+_causal_conv1d_fwd_cpp = torch.ops.DaoAILab._causal_conv1d_fwd_cpp
+_causal_conv1d_bwd_cpp = torch.ops.DaoAILab._causal_conv1d_bwd_cpp
+_causal_conv1d_update_cpp = torch.ops.DaoAILab._causal_conv1d_update_cpp
 
 
 def _states_like(x: Tensor, width: int) -> Tensor:

@@ -9,6 +9,7 @@
 // current HIP stream from c10 and calls the kernel library.  The only memory it
 // allocates is the backward workspace, through the caching allocator.
 #include <torch/extension.h>
+#include <torch/library.h>
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
@@ -289,6 +290,48 @@ void causal_conv1d_varlen_states(const at::Tensor &x, const at::Tensor &cu_seqle
     check_status(cc1d_varlen_states(&p, current_stream()), "causal_conv1d_varlen_states");
 }
 
+// ---- dispatcher entry points -------------------------------------------------------
+// The same three operators as torch.library ops, registered from C++ so that a call from
+// Python goes dispatcher -> kernel without a Python trampoline in between (a Python-defined
+// custom op costs about 8 us of host time per call, more than the decode kernel itself).
+// Names, argument order and the set of written arguments are those of
+// causal_conv1d/cpp_functions.py:11-91 of the reference.
+
+void fwd_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<at::Tensor> &bias,
+            const std::optional<at::Tensor> &seq_idx, const std::optional<at::Tensor> &initial_states,
+            at::Tensor &out, const std::optional<at::Tensor> &final_states_out, bool silu_activation) {
+    std::optional<at::Tensor> fin = final_states_out;
+    causal_conv1d_fwd(x, weight, bias, seq_idx, initial_states, out, fin, silu_activation);
+}
+
+void bwd_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<at::Tensor> &bias,
+            const at::Tensor &dout, const std::optional<at::Tensor> &seq_idx,
+            const std::optional<at::Tensor> &initial_states, const std::optional<at::Tensor> &dfinal_states,
+            at::Tensor &dx, at::Tensor &dweight, const std::optional<at::Tensor> &dbias,
+            const std::optional<at::Tensor> &dinitial_states, bool silu_activation) {
+    at::Tensor dout_ = dout;
+    std::optional<at::Tensor> db = dbias, dinit = dinitial_states;
+    causal_conv1d_bwd(x, weight, bias, dout_, seq_idx, initial_states, dfinal_states, dx, dweight, db, dinit,
+                      silu_activation);
+}
+
+void update_op(const at::Tensor &x, at::Tensor &conv_state, const at::Tensor &weight,
+               const std::optional<at::Tensor> &bias, at::Tensor &out, bool silu_activation,
+               const std::optional<at::Tensor> &cache_seqlens, const std::optional<at::Tensor> &conv_state_indices) {
+    causal_conv1d_update(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices);
+}
+
+// Shape propagation has nothing to do: every output is an argument.
+void fwd_meta(const at::Tensor &, const at::Tensor &, const std::optional<at::Tensor> &,
+              const std::optional<at::Tensor> &, const std::optional<at::Tensor> &, at::Tensor &,
+              const std::optional<at::Tensor> &, bool) {}
+void bwd_meta(const at::Tensor &, const at::Tensor &, const std::optional<at::Tensor> &, const at::Tensor &,
+              const std::optional<at::Tensor> &, const std::optional<at::Tensor> &,
+              const std::optional<at::Tensor> &, at::Tensor &, at::Tensor &, const std::optional<at::Tensor> &,
+              const std::optional<at::Tensor> &, bool) {}
+void update_meta(const at::Tensor &, at::Tensor &, const at::Tensor &, const std::optional<at::Tensor> &,
+                 at::Tensor &, bool, const std::optional<at::Tensor> &, const std::optional<at::Tensor> &) {}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -296,4 +339,30 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("causal_conv1d_bwd", &causal_conv1d_bwd, "Causal conv1d backward");
     m.def("causal_conv1d_update", &causal_conv1d_update, "Causal conv1d update");
     m.def("causal_conv1d_varlen_states", &causal_conv1d_varlen_states, "Varlen final-state gather");
+}
+
+TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {
+    m.def("_causal_conv1d_fwd_cpp(Tensor x, Tensor weight, Tensor? bias, Tensor? seq_idx, "
+          "Tensor? initial_states, Tensor(a!) out, Tensor(b!)? final_states_out, bool silu_activation) -> ()",
+          {at::Tag::pt2_compliant_tag});
+    m.def("_causal_conv1d_bwd_cpp(Tensor x, Tensor weight, Tensor? bias, Tensor dout, Tensor? seq_idx, "
+          "Tensor? initial_states, Tensor(a!)? dfinal_states, Tensor(b!) dx, Tensor(c!) dweight, "
+          "Tensor(d!)? dbias, Tensor(e!)? dinitial_states, bool silu_activation) -> ()",
+          {at::Tag::pt2_compliant_tag});
+    m.def("_causal_conv1d_update_cpp(Tensor x, Tensor(a!) conv_state, Tensor weight, Tensor? bias, "
+          "Tensor(b!) out, bool silu_activation, Tensor? cache_seqlens, Tensor? conv_state_indices) -> ()",
+          {at::Tag::pt2_compliant_tag});
+}
+
+// One kernel for every real backend: on anything but the GPU it raises (there is no host path).
+TORCH_LIBRARY_IMPL(DaoAILab, CompositeExplicitAutograd, m) {
+    m.impl("_causal_conv1d_fwd_cpp", &fwd_op);
+    m.impl("_causal_conv1d_bwd_cpp", &bwd_op);
+    m.impl("_causal_conv1d_update_cpp", &update_op);
+}
+
+TORCH_LIBRARY_IMPL(DaoAILab, Meta, m) {
+    m.impl("_causal_conv1d_fwd_cpp", &fwd_meta);
+    m.impl("_causal_conv1d_bwd_cpp", &bwd_meta);
+    m.impl("_causal_conv1d_update_cpp", &update_meta);
 }
