@@ -268,8 +268,10 @@ def bench_others(ext, dev, steps, warmup):
 
 
 # ------------------------------------------------------------------------ CPU baseline
-def cpu_baseline(cfg_cpu, n_bytes):
-    """The PyTorch oracle on the host, same inputs, whole C2 workload per repetition."""
+def cpu_baseline(cfg_cpu, n_bytes, gpu_out):
+    """The PyTorch oracle on the host, same inputs, whole C2 workload per repetition.  Its
+    result doubles as the check of what the GPU just produced (`gpu_out`, already on the
+    host): this is the only place the benchmark touches the oracle."""
     import torch
     from oracle import causal_conv1d_oracle as orc
     cores = os.cpu_count() or 1
@@ -282,11 +284,14 @@ def cpu_baseline(cfg_cpu, n_bytes):
         t_end = time.perf_counter() + 20.0
         while len(times) < 5 and (len(times) < 2 or time.perf_counter() < t_end):
             t0 = time.perf_counter()
-            orc.fwd_seq_idx(x, w, b, seq, activation="silu")
+            ref = orc.fwd_seq_idx(x, w, b, seq, activation="silu")
             times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
+    err = (gpu_out.float() - ref.float()).abs_()
+    parity_ok = bool(torch.all(err <= 5e-2 + 1e-2 * ref.float().abs()))      # bf16: rtol 1e-2, atol 5e-2
     return {"value": round(n_bytes / med * 1e-9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
             "kind": "port", "us_per_call": round(med * 1e6, 1),
+            "gpu_output_matches": parity_ok, "gpu_max_abs_err": float(err.max()),
             "sample": "the full prefill workload (8 x 5376 x 2048 bf16 + seq_idx), median of %d calls "
                       "of the PyTorch F.conv1d oracle after one warm-up" % len(times)}
 
@@ -294,8 +299,8 @@ def cpu_baseline(cfg_cpu, n_bytes):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--rows", type=int, default=0, help="override rows per lane run (sweeps)")
@@ -334,12 +339,7 @@ def main():
               (nbytes(flat_src), nbytes(flat_dst), copy_us), file=sys.stderr)
         del flat_src, flat_dst
 
-    # Parity of what was just timed, against the oracle on a slice small enough to be quick.
-    from oracle import causal_conv1d_oracle as orc
-    ref = orc.fwd_seq_idx(cfg_cpu["x"][:1], cfg_cpu["weight"], cfg_cpu["bias"], cfg_cpu["seq_idx"][:1], activation="silu")
-    got = out[:1].float().cpu()
-    err = (got - ref.float()).abs()
-    parity_ok = bool(torch.all(err <= 5e-2 + 1e-2 * ref.float().abs()))
+    gpu_out_host = out.cpu()                # checked against the CPU baseline's result below
 
     # End-to-end through the public Python API (allocation + op dispatch included).
     from causal_conv1d import causal_conv1d_fn
@@ -363,8 +363,7 @@ def main():
         "config": {"workload": "Mamba-2 2.7B prefill forward: bf16 x (8, 5376, 2048) channel-last, width 4, "
                                "bias, SiLU, int32 seq_idx with 1-4 packed sub-sequences per row",
                    "algorithmic_bytes": int(n_bytes), "us_per_call": round(us, 3),
-                   "us_per_call_python_api_wall": round(api_wall, 2),
-                   "parity_vs_oracle_ok": parity_ok, "max_abs_err": float(err.max())},
+                   "us_per_call_python_api_wall": round(api_wall, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs(n_bytes, us), 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs(n_bytes, us) / HBM_PEAK_GBS, 4), "traffic": None},
     }
@@ -374,7 +373,7 @@ def main():
             if ln.startswith("traffic_bytes_per_launch:"):
                 line["roofline"]["traffic"] = int(float(ln.split(":")[1]))
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(cfg_cpu, n_bytes)
+        line["cpu_baseline"] = cpu_baseline(cfg_cpu, n_bytes, gpu_out_host)
     del cfg, x, out
     if not args.no_others:
         try:
