@@ -29,12 +29,6 @@ inline bool weights_contiguous_f32(const void *w, int w_dtype, int64_t sc, int64
     return w_dtype == CC1D_F32 && sw == 1 && sc == width && aligned16(w);
 }
 
-// A (batch, dim, k) states tensor can be accessed as 16-byte vectors along dim.
-inline bool states_vec_ok(const void *p, int x_dtype, int64_t sb, int64_t sc, int64_t sl) {
-    const int v = vec_elems(x_dtype);
-    return p != nullptr && sc == 1 && sb % v == 0 && sl % v == 0 && aligned16(p);
-}
-
 struct Tunables {
     int32_t fwd_cl_rows = 0;
     int32_t fwd_cl_half_vec = 0;
