@@ -317,7 +317,10 @@ bool rows_lane_ok(const void *ptr, int dtype, int lane_bytes, int64_t sb, int64_
 }
 
 constexpr int kStepLaneBytes = 8;
-constexpr int kStepRows = 2;
+#ifndef CC1D_UPDATE_STEP_ROWS
+#define CC1D_UPDATE_STEP_ROWS 2
+#endif
+constexpr int kStepRows = CC1D_UPDATE_STEP_ROWS;   // batch rows per lane
 
 template <int DT, int W>
 int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
