@@ -13,6 +13,7 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
+#include <cstdint>
 #include <optional>
 
 #include "cc1d.h"
@@ -30,6 +31,12 @@ int to_cc1d_dtype(at::ScalarType t, const char *what) {
         default: TORCH_CHECK(false, what, " must be float32, float16 or bfloat16, got ", toString(t));
     }
     return -1;
+}
+
+// Sizes travel as int32 in the C ABI; strides and offsets are 64-bit.
+int32_t size32(int64_t v, const char *what) {
+    TORCH_CHECK(v >= 0 && v <= INT32_MAX, what, " = ", v, " does not fit the 32-bit sizes of the kernel library");
+    return static_cast<int32_t>(v);
 }
 
 void check_status(int st, const char *op) {
@@ -64,7 +71,8 @@ void causal_conv1d_fwd(const at::Tensor &x, const at::Tensor &weight,
     check_bias(bias_, weight.scalar_type(), dim);
 
     cc1d_fwd_params p = {};
-    p.batch = (int32_t)batch; p.dim = (int32_t)dim; p.seqlen = (int32_t)seqlen; p.width = (int32_t)width;
+    p.batch = size32(batch, "batch"); p.dim = size32(dim, "dim"); p.seqlen = size32(seqlen, "seqlen");
+    p.width = size32(width, "width");
     p.x_dtype = to_cc1d_dtype(x.scalar_type(), "x");
     p.w_dtype = to_cc1d_dtype(weight.scalar_type(), "weight");
     p.silu = silu_activation ? 1 : 0;
@@ -135,7 +143,8 @@ void causal_conv1d_bwd(const at::Tensor &x, const at::Tensor &weight,
     if (channel_last && dout.stride(1) != 1) dout = dout.transpose(-1, -2).contiguous().transpose(-1, -2);
 
     cc1d_bwd_params p = {};
-    p.batch = (int32_t)batch; p.dim = (int32_t)dim; p.seqlen = (int32_t)seqlen; p.width = (int32_t)width;
+    p.batch = size32(batch, "batch"); p.dim = size32(dim, "dim"); p.seqlen = size32(seqlen, "seqlen");
+    p.width = size32(width, "width");
     p.x_dtype = to_cc1d_dtype(x.scalar_type(), "x");
     p.w_dtype = to_cc1d_dtype(weight.scalar_type(), "weight");
     p.silu = silu_activation ? 1 : 0;
@@ -221,9 +230,10 @@ void causal_conv1d_update(const at::Tensor &x, const at::Tensor &conv_state, con
     check_bias(bias_, weight.scalar_type(), dim);
 
     cc1d_update_params p = {};
-    p.batch = (int32_t)batch; p.dim = (int32_t)dim; p.seqlen = (int32_t)seqlen; p.width = (int32_t)width;
-    p.state_len = (int32_t)state_len;
-    p.state_batch = (int32_t)conv_state.size(0);
+    p.batch = size32(batch, "batch"); p.dim = size32(dim, "dim"); p.seqlen = size32(seqlen, "seqlen");
+    p.width = size32(width, "width");
+    p.state_len = size32(state_len, "state_len");
+    p.state_batch = size32(conv_state.size(0), "conv_state batch");
     p.x_dtype = to_cc1d_dtype(x.scalar_type(), "x");
     p.w_dtype = to_cc1d_dtype(weight.scalar_type(), "weight");
     p.silu = silu_activation ? 1 : 0;
@@ -275,7 +285,7 @@ void causal_conv1d_varlen_states(const at::Tensor &x, const at::Tensor &cu_seqle
     CHECK_SHAPE(states, batch, dim, state_len);
 
     cc1d_varlen_params p = {};
-    p.batch = (int32_t)batch; p.dim = (int32_t)dim; p.state_len = (int32_t)state_len;
+    p.batch = size32(batch, "batch"); p.dim = size32(dim, "dim"); p.state_len = size32(state_len, "state_len");
     p.x_dtype = to_cc1d_dtype(x.scalar_type(), "x");
     p.cu_seqlens_is_int64 = cu_seqlens.scalar_type() == torch::kInt64 ? 1 : 0;
     p.total_tokens = x.size(0);
