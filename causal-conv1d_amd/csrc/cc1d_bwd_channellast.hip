@@ -48,9 +48,12 @@ struct BwdClGeom {
     uint32_t total;           // batch * n_runs * waves_per_row wavefronts
     uint32_t blocks_per_xcd;  // grid size / 8
     int32_t w_fast;           // weights_contiguous_f32
+    int32_t w_mode;           // weights_mode: 0 general loader, 1 / 2 packed taps
 };
 
-template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U>
+// WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
+// through PackedTaps), 0: any layout and type (general loader).
+template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
 __global__ void __launch_bounds__(kBlock, CC1D_BWD_CL_OCC)
 bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws,
                        const int32_t *__restrict__ seq_idx) {
@@ -79,9 +82,12 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
     const bool full = t0 + T <= L;                    // the run lies inside the sequence
     const int last = full ? T - 1 : L - 1 - t0;       // last row of this run, run-relative
 
+    // Packed taps are only requested here and turned into fp32 by fill_windows(), after the
+    // halo rows and the first row groups have been requested as well.
     float wv[CH][W], bv[CH];
-    load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w,
-                        g.w_fast != 0, c0, wv, bv);
+    PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
+    if (WM != 0) taps.request(p.weight, p.bias, c0);
+    else load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, g.w_fast != 0, c0, wv, bv);
 
     // Row pointers of this run; offsets inside a run fit 32 bits (checked by the launcher).
     const char *xrun = reinterpret_cast<const char *>(reinterpret_cast<const T_ *>(p.x) + (int64_t)b * p.x_stride_b + c0 + (int64_t)t0 * p.x_stride_l);
@@ -164,6 +170,7 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
         if (t >= 0) dh_raw[k] = *reinterpret_cast<const raw_t *>(drun - (int64_t)(W - 1 - k) * ds);
     }
     auto fill_windows = [&]() __attribute__((always_inline)) {
+        if (WM != 0) taps.finish(p.bias != nullptr, wv, bv);
         float xh[2 * (W - 1)][CH];
 #pragma unroll
         for (int q = 0; q < 2 * (W - 1); ++q) P::unpack(xh_raw[q], xh[q]);
@@ -470,28 +477,38 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
+    g.w_mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     return true;
 }
 
-template <int DT, int CH, int W, bool HAS_SEQ>
+template <int DT, int CH, int W, bool HAS_SEQ, int WM>
 int launch_instance(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStream_t stream) {
     constexpr int U = CC1D_BWD_CL_UNROLL;
     const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
+        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
     else
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
+        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
     return launch_status();
+}
+
+template <int DT, int CH, int WM>
+int launch_width(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStream_t stream) {
+    const bool seq = p.seq_idx != nullptr;
+    switch (p.width) {
+        case 2: return seq ? launch_instance<DT, CH, 2, true, WM>(p, g, ws, stream) : launch_instance<DT, CH, 2, false, WM>(p, g, ws, stream);
+        case 3: return seq ? launch_instance<DT, CH, 3, true, WM>(p, g, ws, stream) : launch_instance<DT, CH, 3, false, WM>(p, g, ws, stream);
+        default: return seq ? launch_instance<DT, CH, 4, true, WM>(p, g, ws, stream) : launch_instance<DT, CH, 4, false, WM>(p, g, ws, stream);
+    }
 }
 
 template <int DT, int CH>
 int launch_dtype(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStream_t stream) {
-    const bool seq = p.seq_idx != nullptr;
-    switch (p.width) {
-        case 2: return seq ? launch_instance<DT, CH, 2, true>(p, g, ws, stream) : launch_instance<DT, CH, 2, false>(p, g, ws, stream);
-        case 3: return seq ? launch_instance<DT, CH, 3, true>(p, g, ws, stream) : launch_instance<DT, CH, 3, false>(p, g, ws, stream);
-        default: return seq ? launch_instance<DT, CH, 4, true>(p, g, ws, stream) : launch_instance<DT, CH, 4, false>(p, g, ws, stream);
+    if (g.w_mode == 1) return launch_width<DT, CH, 1>(p, g, ws, stream);
+    if constexpr (DT != CC1D_F32) {
+        if (g.w_mode == 2) return launch_width<DT, CH, 2>(p, g, ws, stream);
     }
+    return launch_width<DT, CH, 0>(p, g, ws, stream);
 }
 
 }  // namespace

@@ -274,27 +274,60 @@ __device__ __forceinline__ void load_weights(const void *weight, const void *bia
         bv[j] = bias == nullptr ? 0.f : ld_weight(bias, w_dtype, c0 + j);
 }
 
-// The same for taps and bias known to be fp32, packed (dim, W) and 16-byte aligned: plain
-// vector loads with no branch on the element type and no use of the loaded values, so a
-// caller can issue further loads before it first touches them.  Without a bias, bv holds
-// unspecified finite-or-not bits that the caller must replace by zero.
-template <int W, int NCH>
-__device__ __forceinline__ void load_weights_f32(const void *weight, const void *bias, int c0,
-                                                 float (&wv)[NCH][W], float (&bv)[NCH]) {
-    constexpr int kAlign = NCH * 4 > 16 ? 16 : NCH * 4;
-    const float *src = static_cast<const float *>(__builtin_assume_aligned(
-        reinterpret_cast<const float *>(weight) + (int64_t)c0 * W, kAlign));
+// Taps and bias of NCH adjacent channels stored packed (dim, W) / (dim,) with element type
+// WDT, base pointers 16-byte aligned (a host-checked promise).  request() issues plain vector
+// loads into raw registers and uses none of the values, so a caller can queue further loads
+// behind it; finish() turns the raw bits into fp32.
+template <int W, int NCH, int WDT>
+struct PackedTaps {
+    static constexpr int kN = NCH * W;
+    static constexpr bool k32 = WDT == CC1D_F32;
+    static constexpr int kWords = k32 ? kN : kN / 2;
+    static constexpr int kBiasWords = k32 ? NCH : NCH / 2;
+    uint32_t wraw[kWords];
+    uint32_t braw[kBiasWords];
+    static_assert(NCH % 2 == 0, "two 16-bit taps per word");
+
+    static constexpr int pow2_align(int bytes) { return bytes % 16 == 0 ? 16 : bytes % 8 == 0 ? 8 : 4; }
+
+    __device__ __forceinline__ void request(const void *weight, const void *bias, int c0) {
+        constexpr int kElem = k32 ? 4 : 2;
+        const char *wbase = reinterpret_cast<const char *>(weight) + (int64_t)c0 * W * kElem;
+        const uint32_t *src = static_cast<const uint32_t *>(__builtin_assume_aligned(wbase, pow2_align(kN * kElem)));
 #pragma unroll
-    for (int j = 0; j < NCH; ++j)
+        for (int i = 0; i < kWords; ++i) wraw[i] = src[i];
+        // Without a bias the taps are read a second time in its place: the load stays
+        // unconditional; finish() discards it.
+        const char *bbase = bias != nullptr ? reinterpret_cast<const char *>(bias) + (int64_t)c0 * kElem : wbase;
+        const uint32_t *bsrc = static_cast<const uint32_t *>(__builtin_assume_aligned(bbase, pow2_align(NCH * kElem)));
 #pragma unroll
-        for (int w = 0; w < W; ++w) wv[j][w] = src[j * W + w];
-    // Without a bias the taps are read a second time in its place: the load stays
-    // unconditional and nothing waits for it here.
-    const float *bsrc = bias != nullptr ? reinterpret_cast<const float *>(bias) + c0 : src;
-    bsrc = static_cast<const float *>(__builtin_assume_aligned(bsrc, kAlign));
+        for (int j = 0; j < kBiasWords; ++j) braw[j] = bsrc[j];
+    }
+
+    static __device__ __forceinline__ float element(const uint32_t *words, int i) {
+        if constexpr (k32) {
+            return bitcast<float>(words[i]);
+        } else if constexpr (WDT == CC1D_BF16) {
+            return bitcast<float>(i % 2 ? (words[i / 2] & 0xffff0000u) : (words[i / 2] << 16));
+        } else {
+            const f16x2 h = bitcast<f16x2>(words[i / 2]);
+            return i % 2 ? (float)h.y : (float)h.x;
+        }
+    }
+
+    __device__ __forceinline__ void finish(bool has_bias, float (&wv)[NCH][W], float (&bv)[NCH]) {
+        // Pins the first use of the raw words to this point of the program: without it the
+        // compiler converts them right behind their loads and waits there.
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) bv[j] = bsrc[j];
-}
+        for (int i = 0; i < kWords; ++i) asm volatile("" : "+v"(wraw[i]));
+#pragma unroll
+        for (int j = 0; j < kBiasWords; ++j) asm volatile("" : "+v"(braw[j]));
+#pragma unroll
+        for (int i = 0; i < kN; ++i) wv[i / W][i % W] = element(wraw, i);
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) bv[j] = has_bias ? element(braw, j) : 0.f;
+    }
+};
 
 // ---------------------------------------------------------------------------------
 // Wave64 lane shifts through DPP (no LDS, no memory).  All 64 lanes must be active.

@@ -54,7 +54,9 @@ struct FwdClGeom {
     int32_t w_fast;           // weights_contiguous_f32
 };
 
-template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U>
+// WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
+// through PackedTaps, 8-byte lanes), 0: any layout and type (general loader, 16-byte lanes).
+template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
 __global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CC1D_FWD_CL_OCC8))
 fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t *__restrict__ seq_idx) {
     using E = Elem<DT>;
@@ -81,22 +83,19 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     const int t0 = run * T;                           // < L by construction of n_runs
     const int last = L - 1 - t0;                      // last valid row of this run, run-relative
 
-    // 8-byte lanes exist only for fp32 taps packed (dim, W) (the launcher sees to it): their
-    // loads carry no branch, so everything the run starts with is requested before the first
-    // value is touched.  16-byte lanes take any tap layout and element type.
-    constexpr bool WFAST = CH * E::kBytes == 8;
+    // Packed taps are only requested here: everything the run starts with is in flight before
+    // the first value is touched (prepare() finishes them).
+    constexpr bool WFAST = WM != 0;
     constexpr bool SCALED = SILU && !PRECISE;
     float wv[CH][W], bv[CH];
-    if (WFAST) load_weights_f32<W, CH>(p.weight, p.bias, c0, wv, bv);
+    PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
+    if (WFAST) taps.request(p.weight, p.bias, c0);
     else load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, g.w_fast != 0, c0, wv, bv);
     // 16-bit outputs with SiLU: taps and bias carry the factor -log2(e), so the sums below
     // are already the exponent the activation needs (see silu_from_scaled).  Applied by
     // prepare(), after the first row groups have been requested.
     auto scale_taps = [&]() {
-        if (WFAST && p.bias == nullptr) {
-#pragma unroll
-            for (int j = 0; j < CH; ++j) bv[j] = 0.f;
-        }
+        if (WFAST) taps.finish(p.bias != nullptr, wv, bv);
         if (SCALED) {
 #pragma unroll
             for (int j = 0; j < CH; ++j) {
@@ -318,27 +317,38 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     }
 }
 
-template <int DT, int CH, int W, bool HAS_SEQ>
+template <int DT, int CH, int W, bool HAS_SEQ, int WM>
 int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
     constexpr int U = CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_UNROLL16 : CC1D_FWD_CL_UNROLL;
     const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
-        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U>),
+        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>),
                            dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx);
     else
-        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U>),
+        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>),
                            dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx);
     return launch_status();
 }
 
-template <int DT, int CH>
+template <int DT, int CH, int WM>
 int launch_width(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
     const bool seq = p.seq_idx != nullptr;
     switch (p.width) {
-        case 2: return seq ? launch_instance<DT, CH, 2, true>(p, g, stream) : launch_instance<DT, CH, 2, false>(p, g, stream);
-        case 3: return seq ? launch_instance<DT, CH, 3, true>(p, g, stream) : launch_instance<DT, CH, 3, false>(p, g, stream);
-        default: return seq ? launch_instance<DT, CH, 4, true>(p, g, stream) : launch_instance<DT, CH, 4, false>(p, g, stream);
+        case 2: return seq ? launch_instance<DT, CH, 2, true, WM>(p, g, stream) : launch_instance<DT, CH, 2, false, WM>(p, g, stream);
+        case 3: return seq ? launch_instance<DT, CH, 3, true, WM>(p, g, stream) : launch_instance<DT, CH, 3, false, WM>(p, g, stream);
+        default: return seq ? launch_instance<DT, CH, 4, true, WM>(p, g, stream) : launch_instance<DT, CH, 4, false, WM>(p, g, stream);
     }
+}
+
+// 8-byte lanes with packed taps (mode 1 or 2), else 16-byte lanes with the general loader.
+template <int DT>
+int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, int mode, hipStream_t stream) {
+    constexpr int FULL = Elem<DT>::kVec;
+    if (mode == 1) return launch_width<DT, FULL / 2, 1>(p, g, stream);
+    if constexpr (DT != CC1D_F32) {
+        if (mode == 2) return launch_width<DT, FULL / 2, 2>(p, g, stream);
+    }
+    return launch_width<DT, FULL, 0>(p, g, stream);
 }
 
 }  // namespace
@@ -365,9 +375,9 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
     // 16-byte lane, so twice the waves per SIMD to overlap compute with memory; measured
     // 9% faster at the prefill shape.  fwd_cl_half_vec = -1 selects 16-byte lanes.
     const int full = vec_elems(p.x_dtype);
-    const bool w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width) &&
-                        (p.bias == nullptr || aligned16(p.bias));
-    const int ch = (tunables().fwd_cl_half_vec < 0 || !w_fast) ? full : full / 2;
+    int mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
+    if (tunables().fwd_cl_half_vec < 0) mode = 0;
+    const int ch = mode == 0 ? full : full / 2;
     FwdClGeom g;
     g.n_colgroups = p.dim / ch;
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
@@ -381,11 +391,10 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
-    const bool half = ch != full;
     switch (p.x_dtype) {
-        case CC1D_F32: return half ? launch_width<CC1D_F32, 2>(p, g, stream) : launch_width<CC1D_F32, 4>(p, g, stream);
-        case CC1D_F16: return half ? launch_width<CC1D_F16, 4>(p, g, stream) : launch_width<CC1D_F16, 8>(p, g, stream);
-        default: return half ? launch_width<CC1D_BF16, 4>(p, g, stream) : launch_width<CC1D_BF16, 8>(p, g, stream);
+        case CC1D_F32: return launch_lanes<CC1D_F32>(p, g, mode, stream);
+        case CC1D_F16: return launch_lanes<CC1D_F16>(p, g, mode, stream);
+        default: return launch_lanes<CC1D_BF16>(p, g, mode, stream);
     }
 }
 

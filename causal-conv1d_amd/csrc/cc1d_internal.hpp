@@ -29,6 +29,15 @@ inline bool weights_contiguous_f32(const void *w, int w_dtype, int64_t sc, int64
     return w_dtype == CC1D_F32 && sw == 1 && sc == width && aligned16(w);
 }
 
+// How the fast kernels may read the taps: 1 = packed (dim, width) fp32, 2 = packed in x's own
+// 16-bit type (weight and bias 16-byte aligned, whole vectors per lane, PackedTaps on the
+// device); 0 = anything else (general loader).
+inline int weights_mode(const void *w, const void *bias, int w_dtype, int x_dtype, int64_t sc, int64_t sw, int width) {
+    if (!(sw == 1 && sc == width && aligned16(w) && aligned16(bias))) return 0;
+    if (w_dtype == CC1D_F32) return 1;
+    return w_dtype == x_dtype ? 2 : 0;
+}
+
 struct Tunables {
     int32_t fwd_cl_rows = 0;
     int32_t fwd_cl_half_vec = 0;

@@ -23,6 +23,8 @@
 //   (reads always run ahead of writes, so the shift is safe in place).
 // Circular variant: window = state[(cs-(W-1)+i) mod S], x[i] is written at (cs+i) mod S,
 //   cs = cache_seqlens[b] mod S.
+#include <type_traits>
+
 #include "cc1d_device.hpp"
 #include "cc1d_internal.hpp"
 
@@ -136,8 +138,8 @@ struct StepArgs {
     const void *x;
     void *out;
     void *conv_state;
-    const float *weight;          // fp32, packed (dim, W)
-    const float *bias;            // fp32 or NULL
+    const void *weight;           // packed (dim, W): fp32 or x's own type (template WM)
+    const void *bias;             // same type, or NULL
     const int32_t *cache_seqlens;
     const int32_t *conv_state_indices;
     int64_t x_stride_b, out_stride_b, state_stride_b, state_stride_l;
@@ -146,7 +148,7 @@ struct StepArgs {
 };
 
 // Decode step, one token.  Grid: x = blocks of 256 lanes over dim / CH, y = batch / R.
-template <int DT, int CH, int W, bool CIRC, bool SILU, int R>
+template <int DT, int CH, int W, bool CIRC, bool SILU, int R, int WM>
 __global__ void __launch_bounds__(kBlock)
 update_step_kernel(const StepArgs a) {
     using E = Elem<DT>;
@@ -186,12 +188,10 @@ update_step_kernel(const StepArgs a) {
         }
         xr[r] = *reinterpret_cast<const raw_t *>(xb + (int64_t)bb * a.x_stride_b + c0);
     }
+    PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
+    taps.request(a.weight, a.bias, c0);
     float wv[CH][W], bv[CH];
-    load_weights<W, CH>(a.weight, nullptr, CC1D_F32, W, 1, true, c0, wv, bv);
-    if (a.bias != nullptr) {
-#pragma unroll
-        for (int j = 0; j < CH; ++j) bv[j] = a.bias[c0 + j];
-    }
+    taps.finish(a.bias != nullptr, wv, bv);
 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -326,31 +326,36 @@ template <int DT, int W>
 int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
     const bool circ = p.cache_seqlens != nullptr;
     constexpr int CH = kStepLaneBytes / Elem<DT>::kBytes;
-    // fp32 taps packed (dim, W), as every caller in practice passes them; anything else
-    // takes the general kernels below.
-    const bool step = p.seqlen == 1 && p.dim % CH == 0 && p.batch <= 65535 * kStepRows &&
-        weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width) &&
+    // Taps packed (dim, W) in fp32 or in x's own type, as callers in practice pass them;
+    // anything else takes the general kernels below.
+    const int mode = weights_mode(p.weight, p.bias, p.w_dtype, DT, p.w_stride_c, p.w_stride_w, p.width);
+    const bool step = p.seqlen == 1 && p.dim % CH == 0 && p.batch <= 65535 * kStepRows && mode != 0 &&
         rows_lane_ok(p.x, DT, kStepLaneBytes, p.x_stride_b, p.x_stride_c, p.x_stride_l, 1) &&
         rows_lane_ok(p.out, DT, kStepLaneBytes, p.out_stride_b, p.out_stride_c, p.out_stride_l, 1) &&
         rows_lane_ok(p.conv_state, DT, kStepLaneBytes, p.state_stride_b, p.state_stride_c, p.state_stride_l, p.state_len);
     if (step) {
         StepArgs a;
         a.x = p.x; a.out = p.out; a.conv_state = p.conv_state;
-        a.weight = static_cast<const float *>(p.weight);
-        a.bias = static_cast<const float *>(p.bias);
+        a.weight = p.weight;
+        a.bias = p.bias;
         a.cache_seqlens = p.cache_seqlens; a.conv_state_indices = p.conv_state_indices;
         a.x_stride_b = p.x_stride_b; a.out_stride_b = p.out_stride_b;
         a.state_stride_b = p.state_stride_b; a.state_stride_l = p.state_stride_l;
         a.batch = p.batch; a.state_len = p.state_len;
         a.n_colgroups = (uint32_t)(p.dim / CH);
         const dim3 grid((a.n_colgroups + kBlock - 1) / kBlock, (uint32_t)((p.batch + kStepRows - 1) / kStepRows));
-        if (circ) {
-            if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, true, true, kStepRows>), grid, dim3(kBlock), 0, stream, a);
-            else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, true, false, kStepRows>), grid, dim3(kBlock), 0, stream, a);
-        } else {
-            if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, true, kStepRows>), grid, dim3(kBlock), 0, stream, a);
-            else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, false, kStepRows>), grid, dim3(kBlock), 0, stream, a);
-        }
+        auto launch = [&](auto wm) {
+            constexpr int WM = decltype(wm)::value;
+            if (circ) {
+                if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, true, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+                else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, true, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+            } else {
+                if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+                else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+            }
+        };
+        if (mode == 1) launch(std::integral_constant<int, 1>{});
+        else if constexpr (DT != CC1D_F32) launch(std::integral_constant<int, 2>{});
         return launch_status();
     }
     if (vec) {
