@@ -234,6 +234,116 @@ update_step_kernel(const StepArgs a) {
     }
 }
 
+// A few tokens per call (2 .. kMaxTokens, speculative decoding): one batch row per lane, every
+// x row and the window requested up front under wave-uniform predicates, then the tokens are
+// produced in order from registers.  Grid: x = blocks of 256 lanes over dim / CH, y = batch.
+constexpr int kMaxTokens = 8;
+
+struct TokensArgs {
+    StepArgs s;
+    int64_t x_stride_l, out_stride_l;
+    int32_t seqlen;
+};
+
+template <int DT, int CH, int W, bool CIRC, bool SILU, int WM>
+__global__ void __launch_bounds__(kBlock)
+update_tokens_kernel(const TokensArgs ta) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    using P = Pack<DT, CH>;
+    using raw_t = typename P::raw_t;
+    constexpr bool PRECISE = E::kPreciseAct;
+    const StepArgs &a = ta.s;
+
+    const uint32_t col = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
+    if (col >= a.n_colgroups) return;
+    const int c0 = (int)col * CH;
+    const int b = (int)blockIdx.y;
+    const int S = a.state_len;
+    const int L = ta.seqlen;                          // 2 .. kMaxTokens
+    const T *xrow = reinterpret_cast<const T *>(a.x) + (int64_t)b * a.x_stride_b + c0;
+    T *orow = reinterpret_cast<T *>(a.out) + (int64_t)b * a.out_stride_b + c0;
+
+    const int srow = a.conv_state_indices == nullptr ? b : a.conv_state_indices[b];
+    if (srow < 0) {                                   // padding slot: zeros out, state untouched
+        for (int i = 0; i < L; ++i) *reinterpret_cast<raw_t *>(orow + (int64_t)i * ta.out_stride_l) = P::zero();
+        return;
+    }
+    T *st = reinterpret_cast<T *>(a.conv_state) + (int64_t)srow * a.state_stride_b + c0;
+    int cs = 0;
+    if (CIRC) cs = positive_mod(a.cache_seqlens[b], S);
+
+    raw_t rw[W - 1], xr[kMaxTokens];
+#pragma unroll
+    for (int i = 0; i < W - 1; ++i) {
+        const int l = CIRC ? wrap(cs - (W - 1) + i, S) : S - (W - 1) + i;
+        rw[i] = *reinterpret_cast<const raw_t *>(st + (int64_t)l * a.state_stride_l);
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxTokens; ++i) {
+        xr[i] = P::zero();
+        if (i < L) xr[i] = *reinterpret_cast<const raw_t *>(xrow + (int64_t)i * ta.x_stride_l);
+    }
+    PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
+    taps.request(a.weight, a.bias, c0);
+
+    if (CIRC) {
+        int wpos = cs;
+#pragma unroll
+        for (int i = 0; i < kMaxTokens; ++i) {
+            if (i < L) {
+                *reinterpret_cast<raw_t *>(st + (int64_t)wpos * a.state_stride_l) = xr[i];
+                wpos = wpos + 1 == S ? 0 : wpos + 1;
+            }
+        }
+    } else {
+        // new_state[j] = concat(state, x)[L + j].  Rows in front of the window come from
+        // memory (reads run ahead of writes), window rows and x rows from registers.
+        const int head = S - (W - 1);
+        for (int j = 0; j + L < head; ++j)
+            *reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l) =
+                *reinterpret_cast<const raw_t *>(st + (int64_t)(j + L) * a.state_stride_l);
+#pragma unroll
+        for (int k = 0; k < W - 1; ++k) {
+            const int j = head + k - L;
+            if (j >= 0) *reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l) = rw[k];
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxTokens; ++i) {
+            const int j = S - L + i;
+            if (i < L && j >= 0) *reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l) = xr[i];
+        }
+    }
+
+    float wv[CH][W], bv[CH];
+    taps.finish(a.bias != nullptr, wv, bv);
+    float f[W - 1][CH];
+#pragma unroll
+    for (int k = 0; k < W - 1; ++k) P::unpack(rw[k], f[k]);
+#pragma unroll
+    for (int i = 0; i < kMaxTokens; ++i) {
+        if (i < L) {
+            float xv[CH], acc[CH];
+            P::unpack(xr[i], xv);
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                float z = bv[j];
+#pragma unroll
+                for (int k = 0; k < W - 1; ++k) z = fmaf(wv[j][k], f[k][j], z);
+                z = fmaf(wv[j][W - 1], xv[j], z);
+                acc[j] = SILU ? silu<PRECISE>(z) : z;
+            }
+            *reinterpret_cast<raw_t *>(orow + (int64_t)i * ta.out_stride_l) = P::pack(acc);
+#pragma unroll
+            for (int k = 0; k < W - 2; ++k)
+#pragma unroll
+                for (int j = 0; j < CH; ++j) f[k][j] = f[k + 1][j];
+#pragma unroll
+            for (int j = 0; j < CH; ++j) f[W - 2][j] = xv[j];
+        }
+    }
+}
+
 template <int DT, int W, bool CIRC>
 __global__ void __launch_bounds__(kBlock)
 update_generic_kernel(const cc1d_update_params p, const uint32_t total) {
@@ -352,6 +462,37 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
             } else {
                 if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
                 else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+            }
+        };
+        if (mode == 1) launch(std::integral_constant<int, 1>{});
+        else if constexpr (DT != CC1D_F32) launch(std::integral_constant<int, 2>{});
+        return launch_status();
+    }
+    const bool tokens = p.seqlen >= 2 && p.seqlen <= kMaxTokens && p.dim % CH == 0 && p.batch <= 65535 && mode != 0 &&
+        rows_lane_ok(p.x, DT, kStepLaneBytes, p.x_stride_b, p.x_stride_c, p.x_stride_l, p.seqlen) &&
+        rows_lane_ok(p.out, DT, kStepLaneBytes, p.out_stride_b, p.out_stride_c, p.out_stride_l, p.seqlen) &&
+        rows_lane_ok(p.conv_state, DT, kStepLaneBytes, p.state_stride_b, p.state_stride_c, p.state_stride_l, p.state_len);
+    if (tokens) {
+        TokensArgs ta;
+        StepArgs &a = ta.s;
+        a.x = p.x; a.out = p.out; a.conv_state = p.conv_state;
+        a.weight = p.weight;
+        a.bias = p.bias;
+        a.cache_seqlens = p.cache_seqlens; a.conv_state_indices = p.conv_state_indices;
+        a.x_stride_b = p.x_stride_b; a.out_stride_b = p.out_stride_b;
+        a.state_stride_b = p.state_stride_b; a.state_stride_l = p.state_stride_l;
+        a.batch = p.batch; a.state_len = p.state_len;
+        a.n_colgroups = (uint32_t)(p.dim / CH);
+        ta.x_stride_l = p.x_stride_l; ta.out_stride_l = p.out_stride_l; ta.seqlen = p.seqlen;
+        const dim3 grid((a.n_colgroups + kBlock - 1) / kBlock, (uint32_t)p.batch);
+        auto launch = [&](auto wm) {
+            constexpr int WM = decltype(wm)::value;
+            if (circ) {
+                if (p.silu) hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, true, true, WM>), grid, dim3(kBlock), 0, stream, ta);
+                else hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, true, false, WM>), grid, dim3(kBlock), 0, stream, ta);
+            } else {
+                if (p.silu) hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, false, true, WM>), grid, dim3(kBlock), 0, stream, ta);
+                else hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, false, false, WM>), grid, dim3(kBlock), 0, stream, ta);
             }
         };
         if (mode == 1) launch(std::integral_constant<int, 1>{});

@@ -48,19 +48,21 @@ def test_forward_backward_channel_last(pkg, gpu_device, dtype, w_dtype, has_bias
 @pytest.mark.parametrize("width", [2, 3, 4])
 @pytest.mark.parametrize("has_bias", [False, True])
 @pytest.mark.parametrize("circular", [False, True])
+@pytest.mark.parametrize("seqlen", [1, 3, 8])
 @pytest.mark.parametrize("dtype,w_dtype", PAIRS)
-def test_decode_step(pkg, gpu_device, dtype, w_dtype, circular, has_bias, width):
+def test_decode_step(pkg, gpu_device, dtype, w_dtype, seqlen, circular, has_bias, width):
     dev = gpu_device
     g = gen(100 + width)
     B, D, S = 9, 328, 6
-    x = torch.randn(B, D, generator=g).to(dtype)
+    x = torch.randn(B, D, generator=g).to(dtype) if seqlen == 1 else \
+        torch.randn(B, seqlen, D, generator=g).to(dtype).transpose(1, 2)
     st = torch.randn(B, S, D, generator=g).to(dtype).transpose(1, 2)
     w, b = make_wb(D, width, has_bias, g, w_dtype)
     cs = torch.randint(0, 100, (B,), generator=g, dtype=torch.int32) if circular else None
     st_ref = st.clone()
     ref = orc.update(x, st_ref, w.float(), None if b is None else b.float(), activation="silu", cache_seqlens=cs)
     st_dev = to_dev_like(st, dev)
-    got = pkg.causal_conv1d_update(x.to(dev), st_dev, w.to(dev), None if b is None else b.to(dev), activation="silu",
+    got = pkg.causal_conv1d_update(to_dev_like(x, dev), st_dev, w.to(dev), None if b is None else b.to(dev), activation="silu",
                                    cache_seqlens=None if cs is None else cs.to(dev))
     assert torch.equal(st_dev.cpu(), st_ref), "conv_state must be bit-exact"
     assert_close(got, ref.to(dtype), dtype, "out")
