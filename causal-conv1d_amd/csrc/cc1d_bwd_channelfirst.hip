@@ -20,10 +20,12 @@
 // the other tensors use vectors when they share it, elements otherwise.
 //
 // Two kernels share this design.  The streaming kernel takes rows that are 16-byte aligned
-// and whose length is a whole number of step pairs (every power-of-two seqlen from 1024
-// up): no bounds checks, two register sets in ping-pong, and lane 0's x halo is a separate
-// small load of its own, so the sets do not depend on each other and the loads of the next
-// two steps stay in flight while a step is computed.  The general kernel takes the rest.
+// and a whole number of vectors long (seqlen a multiple of 8, or 4 for fp32): whole 64-vector
+// steps run without bounds checks in two register sets in ping-pong, and lane 0's x halo is a
+// separate small load of its own, so the sets do not depend on each other and the loads of
+// the next two steps stay in flight while a step is computed; an odd step and the partly
+// filled last step of a row are done first, one checked step at a time.  The general kernel
+// takes rows that start off the 16-byte grid.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -351,8 +353,12 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
         const int j_begin = seg * g.vecs_per_seg;
         int j_end = j_begin + g.vecs_per_seg;
         if (j_end > n_vecs) j_end = n_vecs;
-        const int n_steps = (j_end - j_begin) / kWave;            // even, >= 2 (or 0)
-        if (n_steps <= 0) continue;
+        if (j_begin >= j_end) continue;
+        // The item's lowest full steps, an even number of them, go through the ping-pong
+        // pipeline; what is above them (an odd full step, a partly filled last step of the
+        // row) is done first, one checked step at a time.
+        const int n_steps = (j_end - j_begin) / (2 * kWave) * 2;
+        const int j_pipe_end = j_begin + n_steps * kWave;
         const bool row_top = j_end == n_vecs, row_bottom = j_begin == 0;
 
         // g just right of the item: zero past the row's end, else the next segment's first
@@ -361,7 +367,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) carry_g[i] = row_top ? 0.f : rc.g_at(j_end * VEC + i);
 
-        // Step k counts down the row: k = 0 is the item's highest 64 vectors.
+        // Step k counts down the pipeline's range: k = 0 is its highest 64 vectors.
         auto load_step = [&](int k, u32x4 &rx, u32x4 &rd, halo_t &rh) {
             const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;   // first element of the step
             rx = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xr + e0 + lane * VEC));
@@ -369,8 +375,10 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             const int h0 = e0 >= HALO ? e0 - HALO : 0;              // row start: replaced below
             rh = *reinterpret_cast<const halo_t *>(xr + h0);
         };
-        auto compute_step = [&](auto top, auto bottom, int k, const u32x4 &rx, const u32x4 &rd, const halo_t &rh) {
-            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;
+        // top / bottom: compiled in for the steps that can be the item's highest / lowest;
+        // top_rt / bottom_rt say whether this one is, and is the row's end as well.
+        auto compute_at = [&](auto top, auto bottom, auto checked, bool top_rt, bool bottom_rt, int e0, int nvalid,
+                              const u32x4 &rx, const u32x4 &rd, const halo_t &rh) {
             float xf[VEC], gf[VEC], hf[HALO], carry_x[W - 1];
             E::unpack(rx, xf);
             E::unpack(rd, gf);
@@ -378,7 +386,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
 #pragma unroll
             for (int i = 0; i < W - 1; ++i) carry_x[i] = hf[HALO - (W - 1) + i];
             if (decltype(bottom)::value) {
-                if (row_bottom) {
+                if (bottom_rt) {
 #pragma unroll
                     for (int i = 0; i < W - 1; ++i) carry_x[i] = rc.x_at(i - (W - 1));
                 }
@@ -416,7 +424,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
                 dxv[e] = a;
             }
             if (decltype(top)::value) {
-                if (row_top && p.dfinal_states != nullptr && lane == kWave - 1) {
+                if (top_rt && p.dfinal_states != nullptr && lane == nvalid - 1) {
 #pragma unroll
                     for (int i = 0; i < W - 1; ++i)
                         dxv[VEC - (W - 1) + i] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
@@ -424,7 +432,8 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
                                                                                (int64_t)i * p.dfinal_stride_l);
                 }
             }
-            __builtin_nontemporal_store(E::pack(dxv), reinterpret_cast<u32x4 *>(dxr + e0 + lane * VEC));
+            if (!decltype(checked)::value || lane < nvalid)
+                __builtin_nontemporal_store(E::pack(dxv), reinterpret_cast<u32x4 *>(dxr + e0 + lane * VEC));
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 dB += gf[e];
@@ -433,7 +442,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             }
             if (decltype(bottom)::value) {
                 // dinitial_states[i] = dx at position i-(W-1) < 0: only g[0 .. i] reach it.
-                if (row_bottom && p.dinitial_states != nullptr && lane == 0) {
+                if (bottom_rt && p.dinitial_states != nullptr && lane == 0) {
 #pragma unroll
                     for (int i = 0; i < W - 1; ++i) {
                         float a = 0.f;
@@ -444,6 +453,27 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
                     }
                 }
             }
+        };
+
+        // Checked steps above the pipeline's range, highest first.  Lanes past the item's end
+        // read zeros (so their g is zero) and store nothing.
+        for (int js = j_begin + (j_end - j_begin - 1) / kWave * kWave; js >= j_pipe_end; js -= kWave) {
+            const int nvalid = j_end - js < kWave ? j_end - js : kWave;
+            const int e0 = js * VEC;
+            u32x4 rx = {0u, 0u, 0u, 0u}, rd = {0u, 0u, 0u, 0u};
+            if (lane < nvalid) {
+                rx = *reinterpret_cast<const u32x4 *>(xr + e0 + lane * VEC);
+                rd = *reinterpret_cast<const u32x4 *>(dr + e0 + lane * VEC);
+            }
+            const halo_t rh = *reinterpret_cast<const halo_t *>(xr + (e0 >= HALO ? e0 - HALO : 0));
+            compute_at(Yes{}, Yes{}, Yes{}, row_top && js + nvalid == j_end, row_bottom && js == j_begin, e0, nvalid,
+                       rx, rd, rh);
+        }
+        if (n_steps == 0) continue;
+        const bool pipe_top = row_top && j_pipe_end == j_end;      // nothing was done above it
+        auto compute_step = [&](auto top, auto bottom, int k, const u32x4 &rx, const u32x4 &rd, const halo_t &rh) {
+            compute_at(top, bottom, No{}, pipe_top, row_bottom, (j_begin + (n_steps - 1 - k) * kWave) * VEC, kWave,
+                       rx, rd, rh);
         };
 
         // Two register sets in ping-pong; the first and last pair of steps are peeled so the
@@ -499,7 +529,7 @@ bool rows_aligned(const void *base, int64_t stride_b, int64_t stride_c, int vec)
 
 BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
-    const bool streaming = p.seqlen % (2 * kWave * vec) == 0 &&
+    const bool streaming = p.seqlen % vec == 0 &&
                            rows_aligned(p.x, p.x_stride_b, p.x_stride_c, vec) &&
                            rows_aligned(p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
                            rows_aligned(p.dx, p.dx_stride_b, p.dx_stride_c, vec);

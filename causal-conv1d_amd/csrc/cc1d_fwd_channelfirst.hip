@@ -17,10 +17,11 @@
 // layout, csrc/causal_conv1d.cpp:213,228).
 //
 // Two kernels share this design.  The streaming kernel takes rows of x and out that are
-// 16-byte aligned and a whole number of step pairs long (every power-of-two seqlen from
-// 1024 up): no bounds checks, and two register sets in ping-pong keep the loads of the next
-// two steps in flight while a step is computed and stored.  The general kernel takes the
-// rest.
+// 16-byte aligned and a whole number of vectors long (seqlen a multiple of 8, or 4 for
+// fp32): whole 64-vector steps run without bounds checks in two register sets in ping-pong,
+// which keep the loads of the next two groups in flight while a group is computed and stored;
+// what is left over at the end of a segment (an odd group, a partly filled step) takes a
+// checked step.  The general kernel takes rows that start off the 16-byte grid.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -188,9 +189,9 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
     const int j_begin = seg * g.vecs_per_seg;
     int j_end = j_begin + g.vecs_per_seg;
     if (j_end > n_vecs) j_end = n_vecs;
-    const int n_groups = (j_end - j_begin) / (kWave * U);   // groups of U steps: even, >= 2 (or 0)
+    const int n_groups = (j_end - j_begin) / (2 * kWave * U) * 2;   // whole groups of U steps, in pairs
 
-    if (n_groups > 0) {
+    if (j_begin < j_end) {
         float wv[W], bias_v;
 #pragma unroll
         for (int w = 0; w < W; ++w)
@@ -245,32 +246,61 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
         // peeled so the loop is entered in the state its back edge leaves and the wait counts
         // stay exact.
         u32x4 ra[U], rb[U];
-        load_group(0, ra);
-        load_group(1, rb);
-        if (n_groups == 2) {
-            compute_group(0, ra);
-            compute_group(1, rb);
-        } else {
-            compute_group(0, ra);
-            load_group(2, ra);
-            compute_group(1, rb);
-            load_group(3, rb);
-            int k = 2;
+        if (n_groups >= 2) {
+            load_group(0, ra);
+            load_group(1, rb);
+            if (n_groups == 2) {
+                compute_group(0, ra);
+                compute_group(1, rb);
+            } else {
+                compute_group(0, ra);
+                load_group(2, ra);
+                compute_group(1, rb);
+                load_group(3, rb);
+                int k = 2;
 #pragma clang loop unroll(disable)
-            for (; k + 2 < n_groups; k += 2) {
+                for (; k + 2 < n_groups; k += 2) {
+                    compute_group(k, ra);
+                    load_group(k + 2, ra);
+                    compute_group(k + 1, rb);
+                    load_group(k + 3, rb);
+                }
                 compute_group(k, ra);
-                load_group(k + 2, ra);
                 compute_group(k + 1, rb);
-                load_group(k + 3, rb);
             }
-            compute_group(k, ra);
-            compute_group(k + 1, rb);
+        }
+        // Steps the pairs did not cover, the last of them possibly partly filled: lanes past
+        // the segment's end read zeros and store nothing.
+        for (int j0 = j_begin + n_groups * U * kWave; j0 < j_end; j0 += kWave) {
+            const bool mine = j0 + lane < j_end;
+            u32x4 raw = {0u, 0u, 0u, 0u};
+            const int s = (j0 - j_begin) / kWave;
+            if (mine) raw = *reinterpret_cast<const u32x4 *>(xs + s * (kWave * VEC));
+            float xf[VEC];
+            E::unpack(raw, xf);
+            float xx[VEC + W - 1];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) {
+                xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry[i]);
+                carry[i] = read_lane(xf[VEC - (W - 1) + i], kWave - 1);
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xf[e];
+            float acc[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float a = bias_v;
+#pragma unroll
+                for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
+                acc[e] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
+            }
+            if (mine) *reinterpret_cast<u32x4 *>(os + s * (kWave * VEC)) = E::pack(acc);
         }
     }
 
     // final_states[b, c, i] = xpad[L-(W-1)+i], bit-exact copies, by the row's first wave.
     if (p.final_states != nullptr && seg == 0 && lane < W - 1) {
-        const int t = L - (W - 1) + lane;             // >= 0: a streaming row is at least 512 long
+        const int t = L - (W - 1) + lane;             // >= 0: a streaming row holds at least one vector
         st_raw<DT>(p.final_states, (int64_t)b * p.final_stride_b + (int64_t)c * p.final_stride_c +
                                        (int64_t)lane * p.final_stride_l, ld_raw<DT>(p.x, xrow + t));
     }
@@ -306,8 +336,9 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     const int vec = vec_elems(p.x_dtype);
     const bool aligned = aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
                          aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
-    // Steps per register set: two when rows split into whole pairs of two-step groups.
-    const int streaming = !aligned ? 0 : p.seqlen % (4 * kWave * vec) == 0 ? 2 : p.seqlen % (2 * kWave * vec) == 0 ? 1 : 0;
+    // The streaming kernel needs whole vectors (and W-1 <= one vector for final_states);
+    // steps per register set: two once a row has at least eight steps.
+    const int streaming = !(aligned && p.seqlen % vec == 0) ? 0 : p.seqlen >= 8 * kWave * vec ? 2 : 1;
     // Worst case over row alignments: a row may start up to vec-1 elements into its grid.
     const int64_t max_vecs = streaming ? p.seqlen / vec : ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
     const int64_t rows = (int64_t)p.batch * p.dim;

@@ -21,7 +21,7 @@ from oracle import c_oracle
 
 pytestmark = pytest.mark.gpu
 
-SEQLENS = [1, 2, 8, 16, 32, 64, 128, 129, 130, 151, 256, 372, 512, 784, 1024, 1134, 2048, 4096]
+SEQLENS = [1, 2, 8, 16, 32, 64, 128, 129, 130, 151, 256, 372, 512, 784, 1000, 1024, 1134, 1544, 2048, 2568, 4096]
 
 
 def run_gpu(pkg, dev, x, w, b, dout, seq=None, init=None, dfin=None, act=None):

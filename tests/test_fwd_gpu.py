@@ -20,7 +20,7 @@ from oracle import causal_conv1d_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
-SEQLENS = [1, 2, 8, 16, 32, 64, 128, 129, 130, 151, 256, 372, 512, 784, 1024, 1134, 2048, 4096]
+SEQLENS = [1, 2, 8, 16, 32, 64, 128, 129, 130, 151, 256, 372, 512, 784, 1000, 1024, 1134, 1544, 2048, 2568, 4096]
 
 
 def _grid():
