@@ -9,6 +9,7 @@ backward here is always a fixed-order two-stage sum.
   python benchmark_ops.py --op bwd --batch 4 --dim 4096 --seqlen 8192 --dtype fp16 --states
   python benchmark_ops.py --op update --batch 256 --dim 5376 --state-len 8 --circular
   python benchmark_ops.py --op varlen --batch 64 --dim 5376 --seqlen 1024
+  python benchmark_ops.py --op prefill --batch 16 --dim 5376 --seqlen 256
 """
 import argparse
 import gc
@@ -20,7 +21,8 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
 import torch
 
-from causal_conv1d import causal_conv1d_fn, causal_conv1d_update, causal_conv1d_varlen_states
+from causal_conv1d import (causal_conv1d_fn, causal_conv1d_fwd_varlen_states, causal_conv1d_update,
+                           causal_conv1d_varlen_states)
 from causal_conv1d.cpp_functions import causal_conv1d_bwd_function
 
 HBM_PEAK_GBS = 8000.0
@@ -61,7 +63,9 @@ def nbytes(*ts):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--op", choices=["fwd", "bwd", "update", "varlen"], default="fwd")
+    ap.add_argument("--op", choices=["fwd", "bwd", "update", "varlen", "prefill"], default="fwd",
+                    help="prefill: forward over --batch packed sequences plus their varlen final states, as one "
+                         "call and as the two separate calls")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dim", type=int, default=5376)
     ap.add_argument("--seqlen", type=int, default=2048, help="per-sequence length (varlen: mean length)")
@@ -117,6 +121,20 @@ def main():
         fn = lambda: causal_conv1d_update(x, state, weight, bias, activation=act, cache_seqlens=cache)
         per_chan = (1 + (W - 1) + 1 + 1) if a.circular else (1 + S + S + 1)   # x, state reads, state writes, out
         moved = per_chan * B * D * x.element_size() + nbytes(weight, bias, cache)
+    elif a.op == "prefill":
+        S = a.state_len
+        x = torch.randn(1, B * L, D, device=dev, dtype=dtype).transpose(1, 2)
+        cu = torch.arange(B + 1, device=dev, dtype=torch.int32) * L
+        seq = (torch.arange(B * L, device=dev, dtype=torch.int32) // L).reshape(1, B * L)
+        tokens = x[0].t()
+
+        def two_calls():
+            causal_conv1d_fn(x, weight, bias, seq_idx=seq, activation=act)
+            causal_conv1d_varlen_states(tokens, cu, S)
+        with torch.no_grad():
+            print("two calls: %.2f us" % timed(two_calls, a.warmup, a.rep, a.iters))
+        fn = lambda: causal_conv1d_fwd_varlen_states(x, weight, bias, seq, cu, S, activation=act)
+        moved = 2 * nbytes(x) + nbytes(seq, weight, bias, cu) + 2 * B * D * S * x.element_size()
     else:
         S = a.state_len
         lens = torch.randint(max(1, L // 2), L + L // 2, (B,))

@@ -56,7 +56,7 @@ void check_bias(const std::optional<at::Tensor> &bias_, at::ScalarType weight_ty
     CHECK_SHAPE(bias, dim);
 }
 
-void causal_conv1d_fwd(const at::Tensor &x, const at::Tensor &weight,
+cc1d_fwd_params fwd_params(const at::Tensor &x, const at::Tensor &weight,
                        const std::optional<at::Tensor> &bias_,
                        const std::optional<at::Tensor> &seq_idx_,
                        const std::optional<at::Tensor> &initial_states_, at::Tensor &out,
@@ -109,6 +109,16 @@ void causal_conv1d_fwd(const at::Tensor &x, const at::Tensor &weight,
         p.final_stride_b = s.stride(0); p.final_stride_c = s.stride(1); p.final_stride_l = s.stride(2);
     }
 
+    return p;
+}
+
+void causal_conv1d_fwd(const at::Tensor &x, const at::Tensor &weight,
+                       const std::optional<at::Tensor> &bias_,
+                       const std::optional<at::Tensor> &seq_idx_,
+                       const std::optional<at::Tensor> &initial_states_, at::Tensor &out,
+                       std::optional<at::Tensor> &final_states_out_, bool silu_activation) {
+    const cc1d_fwd_params p = fwd_params(x, weight, bias_, seq_idx_, initial_states_, out, final_states_out_,
+                                         silu_activation);
     c10::DeviceGuard device_guard(x.device());   // otherwise the launch lands on device 0
     check_status(cc1d_fwd(&p, current_stream()), "causal_conv1d_fwd");
 }
@@ -272,7 +282,7 @@ void causal_conv1d_update(const at::Tensor &x, const at::Tensor &conv_state, con
     check_status(cc1d_update(&p, current_stream()), "causal_conv1d_update");
 }
 
-void causal_conv1d_varlen_states(const at::Tensor &x, const at::Tensor &cu_seqlens, at::Tensor &states,
+cc1d_varlen_params varlen_params(const at::Tensor &x, const at::Tensor &cu_seqlens, at::Tensor &states,
                                  int64_t state_len) {
     TORCH_CHECK(x.is_cuda() && cu_seqlens.is_cuda() && states.is_cuda(), "tensors must be on the GPU");
     TORCH_CHECK(x.dim() == 2, "x must be (total_tokens, dim)");
@@ -296,8 +306,30 @@ void causal_conv1d_varlen_states(const at::Tensor &x, const at::Tensor &cu_seqle
     p.states_stride_b = states.stride(0); p.states_stride_c = states.stride(1);
     p.states_stride_l = states.stride(2);
 
+    return p;
+}
+
+void causal_conv1d_varlen_states(const at::Tensor &x, const at::Tensor &cu_seqlens, at::Tensor &states,
+                                 int64_t state_len) {
+    const cc1d_varlen_params p = varlen_params(x, cu_seqlens, states, state_len);
     c10::DeviceGuard device_guard(x.device());
     check_status(cc1d_varlen_states(&p, current_stream()), "causal_conv1d_varlen_states");
+}
+
+// Forward over a packed batch and the gather of every sequence's last state_len tokens from
+// `tokens` (total_tokens, dim), normally a view of x: one call, and one kernel launch when x is
+// channel-last.  What causal_conv1d_fwd followed by causal_conv1d_varlen_states would give.
+void causal_conv1d_fwd_varlen_states(const at::Tensor &x, const at::Tensor &weight,
+                                     const std::optional<at::Tensor> &bias_,
+                                     const std::optional<at::Tensor> &seq_idx_, at::Tensor &out,
+                                     const at::Tensor &tokens, const at::Tensor &cu_seqlens,
+                                     at::Tensor &states, int64_t state_len, bool silu_activation) {
+    std::optional<at::Tensor> none;
+    const cc1d_fwd_params f = fwd_params(x, weight, bias_, seq_idx_, none, out, none, silu_activation);
+    const cc1d_varlen_params v = varlen_params(tokens, cu_seqlens, states, state_len);
+    TORCH_CHECK(tokens.device() == x.device(), "tokens must be on the device of x");
+    c10::DeviceGuard device_guard(x.device());
+    check_status(cc1d_fwd_varlen_states(&f, &v, current_stream()), "causal_conv1d_fwd_varlen_states");
 }
 
 // ---- dispatcher entry points -------------------------------------------------------
@@ -349,6 +381,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("causal_conv1d_bwd", &causal_conv1d_bwd, "Causal conv1d backward");
     m.def("causal_conv1d_update", &causal_conv1d_update, "Causal conv1d update");
     m.def("causal_conv1d_varlen_states", &causal_conv1d_varlen_states, "Varlen final-state gather");
+    m.def("causal_conv1d_fwd_varlen_states", &causal_conv1d_fwd_varlen_states,
+          "Causal conv1d forward and varlen final-state gather in one call");
 }
 
 TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {

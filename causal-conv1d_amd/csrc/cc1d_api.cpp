@@ -139,8 +139,27 @@ int cc1d_fwd(const cc1d_fwd_params *p, cc1d_stream_t stream) {
     if (st != CC1D_OK) return st;
     if (is_empty(p)) return CC1D_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return is_channel_last(p->x_stride_c, p->x_stride_l) ? launch_fwd_channellast(*p, s)
+    return is_channel_last(p->x_stride_c, p->x_stride_l) ? launch_fwd_channellast(*p, nullptr, s)
                                                          : launch_fwd_channelfirst(*p, s);
+}
+
+int cc1d_fwd_varlen_states(const cc1d_fwd_params *fwd, const cc1d_varlen_params *gather, cc1d_stream_t stream) {
+    int st = cc1d_validate_fwd(fwd);
+    if (st != CC1D_OK) return st;
+    st = cc1d_validate_varlen_states(gather);
+    if (st != CC1D_OK) return st;
+    const bool no_gather = gather->batch == 0 || gather->dim == 0 || gather->state_len == 0;
+    if (is_empty(fwd) || no_gather) {
+        st = cc1d_fwd(fwd, stream);
+        return st != CC1D_OK ? st : cc1d_varlen_states(gather, stream);
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // One launch when the forward is channel-last and the gather moves whole 16-byte vectors
+    // of elements as wide as the forward's; two launches otherwise.
+    if (is_channel_last(fwd->x_stride_c, fwd->x_stride_l) && varlen_fits_fwd_launch(*fwd, *gather))
+        return launch_fwd_channellast(*fwd, gather, s);
+    st = cc1d_fwd(fwd, stream);
+    return st != CC1D_OK ? st : launch_varlen_states(*gather, s);
 }
 
 // ------------------------------------------------------------------------ backward

@@ -20,8 +20,7 @@
 // with the normal cache policy while everything else streams through (non-temporal).
 #include <type_traits>
 
-#include "cc1d_device.hpp"
-#include "cc1d_internal.hpp"
+#include "cc1d_varlen_gather.hpp"
 
 // Rows per register set; two sets are in flight per lane.
 #ifndef CC1D_FWD_CL_UNROLL
@@ -58,13 +57,21 @@ struct FwdClGeom {
 // through PackedTaps, 8-byte lanes), 0: any layout and type (general loader, 16-byte lanes).
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
 __global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CC1D_FWD_CL_OCC8))
-fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t *__restrict__ seq_idx) {
+fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t *__restrict__ seq_idx,
+                       const VarlenTail tail) {
     using E = Elem<DT>;
     using T_ = typename E::type;
     using P = Pack<DT, CH>;
     using raw_t = typename P::raw_t;
     constexpr bool PRECISE = E::kPreciseAct;
 
+    // Workgroups past the forward's own are there for the varlen final-state gather, which
+    // reads x only and so needs no ordering against the rows being produced.
+    if (blockIdx.x >= tail.first_block) {
+        varlen_gather_vec<DT>(tail.p, tail.n_colgroups, tail.total,
+                              (blockIdx.x - tail.first_block) * (uint32_t)kBlock + threadIdx.x);
+        return;
+    }
     // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
     const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
     // A wavefront never straddles two runs: its batch index, run and row range are scalars,
@@ -318,37 +325,37 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
 }
 
 template <int DT, int CH, int W, bool HAS_SEQ, int WM>
-int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
+int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail &tail, hipStream_t stream) {
     constexpr int U = CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_UNROLL16 : CC1D_FWD_CL_UNROLL;
-    const uint32_t blocks = g.blocks_per_xcd * kXcds;
+    const uint32_t blocks = tail.first_block + (tail.total + kBlock - 1) / kBlock;
     if (p.silu)
         hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>),
-                           dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx);
+                           dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx, tail);
     else
         hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>),
-                           dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx);
+                           dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx, tail);
     return launch_status();
 }
 
 template <int DT, int CH, int WM>
-int launch_width(const cc1d_fwd_params &p, const FwdClGeom &g, hipStream_t stream) {
+int launch_width(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail &tail, hipStream_t stream) {
     const bool seq = p.seq_idx != nullptr;
     switch (p.width) {
-        case 2: return seq ? launch_instance<DT, CH, 2, true, WM>(p, g, stream) : launch_instance<DT, CH, 2, false, WM>(p, g, stream);
-        case 3: return seq ? launch_instance<DT, CH, 3, true, WM>(p, g, stream) : launch_instance<DT, CH, 3, false, WM>(p, g, stream);
-        default: return seq ? launch_instance<DT, CH, 4, true, WM>(p, g, stream) : launch_instance<DT, CH, 4, false, WM>(p, g, stream);
+        case 2: return seq ? launch_instance<DT, CH, 2, true, WM>(p, g, tail, stream) : launch_instance<DT, CH, 2, false, WM>(p, g, tail, stream);
+        case 3: return seq ? launch_instance<DT, CH, 3, true, WM>(p, g, tail, stream) : launch_instance<DT, CH, 3, false, WM>(p, g, tail, stream);
+        default: return seq ? launch_instance<DT, CH, 4, true, WM>(p, g, tail, stream) : launch_instance<DT, CH, 4, false, WM>(p, g, tail, stream);
     }
 }
 
 // 8-byte lanes with packed taps (mode 1 or 2), else 16-byte lanes with the general loader.
 template <int DT>
-int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, int mode, hipStream_t stream) {
+int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail &tail, int mode, hipStream_t stream) {
     constexpr int FULL = Elem<DT>::kVec;
-    if (mode == 1) return launch_width<DT, FULL / 2, 1>(p, g, stream);
+    if (mode == 1) return launch_width<DT, FULL / 2, 1>(p, g, tail, stream);
     if constexpr (DT != CC1D_F32) {
-        if (mode == 2) return launch_width<DT, FULL / 2, 2>(p, g, stream);
+        if (mode == 2) return launch_width<DT, FULL / 2, 2>(p, g, tail, stream);
     }
-    return launch_width<DT, FULL, 0>(p, g, stream);
+    return launch_width<DT, FULL, 0>(p, g, tail, stream);
 }
 
 }  // namespace
@@ -370,7 +377,9 @@ static int choose_rows_per_run(int seqlen, int64_t row_bytes) {
     return (int64_t)T * row_bytes >= ((int64_t)1 << 31) ? 0 : T;
 }
 
-int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
+// gather: a varlen final-state gather to run in the same launch (NULL: none).  It must be one
+// the vector gather takes (varlen_vec_ok) on elements as wide as x's.
+int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *gather, hipStream_t stream) {
     // Channels per lane: an 8-byte vector (4 x 16-bit or 2 x fp32).  Half the registers of a
     // 16-byte lane, so twice the waves per SIMD to overlap compute with memory; measured
     // 9% faster at the prefill shape.  fwd_cl_half_vec = -1 selects 16-byte lanes.
@@ -391,10 +400,19 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream) {
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
+    VarlenTail tail = {};
+    tail.first_block = g.blocks_per_xcd * kXcds;
+    if (gather != nullptr) {
+        tail.p = *gather;
+        tail.n_colgroups = (uint32_t)(gather->dim / vec_elems(gather->x_dtype));
+        const int64_t threads = (int64_t)gather->batch * gather->state_len * tail.n_colgroups;
+        if (threads + (int64_t)tail.first_block * kBlock >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+        tail.total = (uint32_t)threads;
+    }
     switch (p.x_dtype) {
-        case CC1D_F32: return launch_lanes<CC1D_F32>(p, g, mode, stream);
-        case CC1D_F16: return launch_lanes<CC1D_F16>(p, g, mode, stream);
-        default: return launch_lanes<CC1D_BF16>(p, g, mode, stream);
+        case CC1D_F32: return launch_lanes<CC1D_F32>(p, g, tail, mode, stream);
+        case CC1D_F16: return launch_lanes<CC1D_F16>(p, g, tail, mode, stream);
+        default: return launch_lanes<CC1D_BF16>(p, g, tail, mode, stream);
     }
 }
 

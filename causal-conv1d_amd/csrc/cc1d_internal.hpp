@@ -38,6 +38,20 @@ inline int weights_mode(const void *w, const void *bias, int w_dtype, int x_dtyp
     return w_dtype == x_dtype ? 2 : 0;
 }
 
+// Varlen gather: x and states have unit stride along dim and every vector is 16-byte aligned.
+inline bool varlen_vec_ok(const cc1d_varlen_params &p) {
+    const int v = vec_elems(p.x_dtype);
+    return p.dim % v == 0 && p.x_stride_c == 1 && p.x_stride_t % v == 0 && aligned16(p.x) &&
+           p.states_stride_c == 1 && p.states_stride_b % v == 0 &&
+           (p.state_len <= 1 || p.states_stride_l % v == 0) && aligned16(p.states);
+}
+
+// The gather can ride in the channel-last forward's launch: vector copies of elements as
+// wide as the forward's.
+inline bool varlen_fits_fwd_launch(const cc1d_fwd_params &f, const cc1d_varlen_params &v) {
+    return varlen_vec_ok(v) && elem_bytes(v.x_dtype) == elem_bytes(f.x_dtype);
+}
+
 struct Tunables {
     int32_t fwd_cl_rows = 0;
     int32_t fwd_cl_half_vec = 0;
@@ -51,7 +65,7 @@ inline int launch_status() {
     return hipGetLastError() == hipSuccess ? CC1D_OK : CC1D_ERR_LAUNCH;
 }
 
-int launch_fwd_channellast(const cc1d_fwd_params &p, hipStream_t stream);
+int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *gather, hipStream_t stream);
 int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream);
 
 size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p);

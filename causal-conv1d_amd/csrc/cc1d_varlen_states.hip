@@ -9,42 +9,16 @@
 // of channels of one (sequence, state column) when x and states have unit stride along
 // dim; any other strides take the element kernel.  Rows that cu_seqlens would place
 // outside [0, total_tokens) are written as zeros instead of being read.
-#include "cc1d_device.hpp"
-#include "cc1d_internal.hpp"
+#include "cc1d_varlen_gather.hpp"
 
 namespace cc1d {
 namespace {
-
-__device__ __forceinline__ int64_t cu_at(const void *cu, bool is64, int i) {
-    return is64 ? reinterpret_cast<const int64_t *>(cu)[i]
-                : (int64_t) reinterpret_cast<const int32_t *>(cu)[i];
-}
-
-// Source row of state column s of sequence b, or -1 for a zero column.
-__device__ __forceinline__ int64_t source_row(const cc1d_varlen_params &p, int b, int s) {
-    const bool is64 = p.cu_seqlens_is_int64 != 0;
-    const int64_t end = cu_at(p.cu_seqlens, is64, b + 1);
-    int64_t start = cu_at(p.cu_seqlens, is64, b);
-    if (start < end - p.state_len) start = end - p.state_len;
-    const int64_t row = end - (p.state_len - s);
-    return (row >= start && row >= 0 && row < p.total_tokens) ? row : -1;
-}
 
 template <int DT>
 __global__ void __launch_bounds__(kBlock)
 varlen_states_vec_kernel(const cc1d_varlen_params p, const uint32_t n_colgroups,
                          const uint32_t total) {
-    constexpr int VEC = Elem<DT>::kVec;
-    const uint32_t gid = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
-    if (gid >= total) return;
-    const int c0 = (int)(gid % n_colgroups) * VEC;
-    const uint32_t bs = gid / n_colgroups;
-    const int s = (int)(bs % (uint32_t)p.state_len);
-    const int b = (int)(bs / (uint32_t)p.state_len);
-    const int64_t row = source_row(p, b, s);
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (row >= 0) v = ld_vec<DT>(p.x, row * p.x_stride_t + c0);
-    st_vec<DT>(p.states, (int64_t)b * p.states_stride_b + (int64_t)s * p.states_stride_l + c0, v);
+    varlen_gather_vec<DT>(p, n_colgroups, total, blockIdx.x * (uint32_t)kBlock + threadIdx.x);
 }
 
 template <int DT>
@@ -84,10 +58,7 @@ int launch_dtype(const cc1d_varlen_params &p, bool vec, hipStream_t stream) {
 }  // namespace
 
 int launch_varlen_states(const cc1d_varlen_params &p, hipStream_t stream) {
-    const int v = vec_elems(p.x_dtype);
-    const bool vec = p.dim % v == 0 && p.x_stride_c == 1 && p.x_stride_t % v == 0 && aligned16(p.x) &&
-                     p.states_stride_c == 1 && p.states_stride_b % v == 0 &&
-                     (p.state_len <= 1 || p.states_stride_l % v == 0) && aligned16(p.states);
+    const bool vec = varlen_vec_ok(p);
     // 2-byte types only differ in how bits are interpreted; the copy treats them alike.
     return p.x_dtype == CC1D_F32 ? launch_dtype<CC1D_F32>(p, vec, stream)
                                  : launch_dtype<CC1D_F16>(p, vec, stream);

@@ -211,6 +211,18 @@ typedef struct cc1d_varlen_params {
 int cc1d_validate_varlen_states(const cc1d_varlen_params *p);
 int cc1d_varlen_states(const cc1d_varlen_params *p, cc1d_stream_t stream);
 
+/* Forward and gather together: what a varlen prefill -> decode hand-off issues back to back,
+ * causal_conv1d_fn over the packed batch (causal_conv1d/causal_conv1d_interface.py:99-129) and
+ * causal_conv1d_varlen_states on the same tokens (causal_conv1d/causal_conv1d_varlen.py:35-64);
+ * the reference has no single call for the pair.  Results are those of cc1d_fwd followed by
+ * cc1d_varlen_states.  The gather reads only its own x, so it does not wait for the forward:
+ * with a channel-last forward and a gather whose x and states have unit stride along dim
+ * (16-byte aligned rows, same element size as the forward's x) both run in ONE kernel launch,
+ * the gather in extra workgroups at the end of the forward's grid; any other combination is
+ * two launches on `stream`.  `gather->states` must not overlap anything the forward writes. */
+int cc1d_fwd_varlen_states(const cc1d_fwd_params *fwd, const cc1d_varlen_params *gather,
+                           cc1d_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Misc.
  * ---------------------------------------------------------------------------------- */

@@ -153,6 +153,7 @@ def declare(lib):
     lib.cc1d_bwd.argtypes = [C.POINTER(BwdParams), vp, C.c_size_t, vp]
     lib.cc1d_update.argtypes = [C.POINTER(UpdateParams), vp]
     lib.cc1d_varlen_states.argtypes = [C.POINTER(VarlenParams), vp]
+    lib.cc1d_fwd_varlen_states.argtypes = [C.POINTER(FwdParams), C.POINTER(VarlenParams), vp]
     lib.cc1d_set_tunable.argtypes = [C.c_char_p, i32]
     lib.cc1d_get_tunable.argtypes = [C.c_char_p, C.POINTER(i32)]
     return lib
