@@ -22,6 +22,9 @@ _Opt = Optional[Tensor]
 _causal_conv1d_fwd_cpp = torch.ops.DaoAILab._causal_conv1d_fwd_cpp
 _causal_conv1d_bwd_cpp = torch.ops.DaoAILab._causal_conv1d_bwd_cpp
 _causal_conv1d_update_cpp = torch.ops.DaoAILab._causal_conv1d_update_cpp
+# Not an op of the reference: the backward with dweight / dbias as plain outputs, so that the
+# wrapper below does not have to zero-fill them first (two small launches per backward call).
+_causal_conv1d_bwd_overwrite_cpp = torch.ops.DaoAILab._causal_conv1d_bwd_overwrite_cpp
 
 
 def _states_like(x: Tensor, width: int) -> Tensor:
@@ -46,14 +49,15 @@ def causal_conv1d_bwd_function(x: Tensor, weight: Tensor, bias: _Opt, dout: Tens
                                initial_states: _Opt, dfinal_states: _Opt, dx: _Opt,
                                return_dinitial_states: bool, silu_activation: bool) -> Tuple[_Opt, ...]:
     """Returns (dx, dweight, dbias, dinitial_states).  dx may be supplied by the caller; dweight
-    and dbias are accumulated in fp32 buffers that start at zero (the kernels add into them)
-    and come back in the parameters' dtype."""
+    and dbias are summed in fp32 (one buffer for both) and come back in the parameters' dtype."""
     dx = torch.empty_like(x) if dx is None else dx
-    dweight32 = torch.zeros_like(weight, dtype=torch.float32)
-    dbias32 = None if bias is None else torch.zeros_like(bias, dtype=torch.float32)
-    dinitial_states = _states_like(x, weight.shape[-1]) if return_dinitial_states else None
-    _causal_conv1d_bwd_cpp(x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
-                           dx, dweight32, dbias32, dinitial_states, silu_activation)
+    dim, width = weight.shape
+    sums = torch.empty(dim * (width + (0 if bias is None else 1)), dtype=torch.float32, device=x.device)
+    dweight32 = sums[:dim * width].view(dim, width)
+    dbias32 = None if bias is None else sums[dim * width:]
+    dinitial_states = _states_like(x, width) if return_dinitial_states else None
+    _causal_conv1d_bwd_overwrite_cpp(x, weight, bias, dout, seq_idx, initial_states, dfinal_states,
+                                     dx, dweight32, dbias32, dinitial_states, silu_activation)
     dbias = None if dbias32 is None else dbias32.type_as(bias)
     return dx, dweight32.type_as(weight), dbias, dinitial_states
 

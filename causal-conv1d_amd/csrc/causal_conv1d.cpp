@@ -123,13 +123,15 @@ void causal_conv1d_fwd(const at::Tensor &x, const at::Tensor &weight,
     check_status(cc1d_fwd(&p, current_stream()), "causal_conv1d_fwd");
 }
 
-void causal_conv1d_bwd(const at::Tensor &x, const at::Tensor &weight,
-                       const std::optional<at::Tensor> &bias_, at::Tensor &dout,
-                       const std::optional<at::Tensor> &seq_idx_,
-                       const std::optional<at::Tensor> &initial_states_,
-                       const std::optional<at::Tensor> &dfinal_states_, at::Tensor &dx,
-                       at::Tensor &dweight, std::optional<at::Tensor> &dbias_,
-                       std::optional<at::Tensor> &dinitial_states_, bool silu_activation) {
+// overwrite = false: dweight / dbias are added into, as in the reference; true: they are plain
+// outputs and may come in uninitialised.
+void bwd_impl(const at::Tensor &x, const at::Tensor &weight,
+              const std::optional<at::Tensor> &bias_, at::Tensor &dout,
+              const std::optional<at::Tensor> &seq_idx_,
+              const std::optional<at::Tensor> &initial_states_,
+              const std::optional<at::Tensor> &dfinal_states_, at::Tensor &dx,
+              at::Tensor &dweight, std::optional<at::Tensor> &dbias_,
+              std::optional<at::Tensor> &dinitial_states_, bool silu_activation, bool overwrite) {
     TORCH_CHECK(x.is_cuda() && weight.is_cuda() && dout.is_cuda() && dx.is_cuda() && dweight.is_cuda(),
                 "tensors must be on the GPU");
     TORCH_CHECK(bias_.has_value() == dbias_.has_value(), "bias and dbias must be given together");
@@ -158,6 +160,7 @@ void causal_conv1d_bwd(const at::Tensor &x, const at::Tensor &weight,
     p.x_dtype = to_cc1d_dtype(x.scalar_type(), "x");
     p.w_dtype = to_cc1d_dtype(weight.scalar_type(), "weight");
     p.silu = silu_activation ? 1 : 0;
+    p.overwrite_dweight = overwrite ? 1 : 0;
     p.x = x.data_ptr();
     p.x_stride_b = x.stride(0); p.x_stride_c = x.stride(1); p.x_stride_l = x.stride(2);
     p.weight = weight.data_ptr();
@@ -219,6 +222,17 @@ void causal_conv1d_bwd(const at::Tensor &x, const at::Tensor &weight,
         ws_ptr = workspace.data_ptr();
     }
     check_status(cc1d_bwd(&p, ws_ptr, ws_bytes, current_stream()), "causal_conv1d_bwd");
+}
+
+void causal_conv1d_bwd(const at::Tensor &x, const at::Tensor &weight,
+                       const std::optional<at::Tensor> &bias_, at::Tensor &dout,
+                       const std::optional<at::Tensor> &seq_idx_,
+                       const std::optional<at::Tensor> &initial_states_,
+                       const std::optional<at::Tensor> &dfinal_states_, at::Tensor &dx,
+                       at::Tensor &dweight, std::optional<at::Tensor> &dbias_,
+                       std::optional<at::Tensor> &dinitial_states_, bool silu_activation) {
+    bwd_impl(x, weight, bias_, dout, seq_idx_, initial_states_, dfinal_states_, dx, dweight, dbias_,
+             dinitial_states_, silu_activation, false);
 }
 
 void causal_conv1d_update(const at::Tensor &x, const at::Tensor &conv_state, const at::Tensor &weight,
@@ -357,6 +371,20 @@ void bwd_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<a
                       silu_activation);
 }
 
+// The backward with dweight / dbias as plain outputs (no zero-fill before the call): what the
+// autograd function of this package uses.  Not an op of the reference.
+void bwd_overwrite_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<at::Tensor> &bias,
+                      const at::Tensor &dout, const std::optional<at::Tensor> &seq_idx,
+                      const std::optional<at::Tensor> &initial_states,
+                      const std::optional<at::Tensor> &dfinal_states, at::Tensor &dx, at::Tensor &dweight,
+                      const std::optional<at::Tensor> &dbias, const std::optional<at::Tensor> &dinitial_states,
+                      bool silu_activation) {
+    at::Tensor dout_ = dout;
+    std::optional<at::Tensor> db = dbias, dinit = dinitial_states;
+    bwd_impl(x, weight, bias, dout_, seq_idx, initial_states, dfinal_states, dx, dweight, db, dinit,
+             silu_activation, true);
+}
+
 void update_op(const at::Tensor &x, at::Tensor &conv_state, const at::Tensor &weight,
                const std::optional<at::Tensor> &bias, at::Tensor &out, bool silu_activation,
                const std::optional<at::Tensor> &cache_seqlens, const std::optional<at::Tensor> &conv_state_indices) {
@@ -393,6 +421,10 @@ TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {
           "Tensor? initial_states, Tensor(a!)? dfinal_states, Tensor(b!) dx, Tensor(c!) dweight, "
           "Tensor(d!)? dbias, Tensor(e!)? dinitial_states, bool silu_activation) -> ()",
           {at::Tag::pt2_compliant_tag});
+    m.def("_causal_conv1d_bwd_overwrite_cpp(Tensor x, Tensor weight, Tensor? bias, Tensor dout, Tensor? seq_idx, "
+          "Tensor? initial_states, Tensor(a!)? dfinal_states, Tensor(b!) dx, Tensor(c!) dweight, "
+          "Tensor(d!)? dbias, Tensor(e!)? dinitial_states, bool silu_activation) -> ()",
+          {at::Tag::pt2_compliant_tag});
     m.def("_causal_conv1d_update_cpp(Tensor x, Tensor(a!) conv_state, Tensor weight, Tensor? bias, "
           "Tensor(b!) out, bool silu_activation, Tensor? cache_seqlens, Tensor? conv_state_indices) -> ()",
           {at::Tag::pt2_compliant_tag});
@@ -402,11 +434,13 @@ TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {
 TORCH_LIBRARY_IMPL(DaoAILab, CompositeExplicitAutograd, m) {
     m.impl("_causal_conv1d_fwd_cpp", &fwd_op);
     m.impl("_causal_conv1d_bwd_cpp", &bwd_op);
+    m.impl("_causal_conv1d_bwd_overwrite_cpp", &bwd_overwrite_op);
     m.impl("_causal_conv1d_update_cpp", &update_op);
 }
 
 TORCH_LIBRARY_IMPL(DaoAILab, Meta, m) {
     m.impl("_causal_conv1d_fwd_cpp", &fwd_meta);
     m.impl("_causal_conv1d_bwd_cpp", &bwd_meta);
+    m.impl("_causal_conv1d_bwd_overwrite_cpp", &bwd_meta);
     m.impl("_causal_conv1d_update_cpp", &update_meta);
 }

@@ -203,7 +203,12 @@ int cc1d_bwd(const cc1d_bwd_params *p, void *workspace, size_t workspace_bytes, 
     size_t need = 0;
     const int st = cc1d_bwd_workspace_bytes(p, &need);
     if (st != CC1D_OK) return st;
-    if (is_empty(p)) return CC1D_OK;
+    if (is_empty(p)) {
+        // Nothing to sum: with overwrite_dweight the outputs still have to become zeros.
+        if (p->overwrite_dweight != 0 && p->dim > 0 && p->dweight != nullptr)
+            return launch_bwd_finalize(nullptr, 0, *p, static_cast<hipStream_t>(stream));
+        return CC1D_OK;
+    }
     if (need > 0 && (workspace == nullptr || !aligned16(workspace) || workspace_bytes < need))
         return CC1D_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);

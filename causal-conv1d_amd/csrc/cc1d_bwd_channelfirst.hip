@@ -34,6 +34,11 @@
 namespace cc1d {
 namespace {
 
+// dweight / dbias are added into unless the caller asked for plain stores.
+__device__ __forceinline__ void accumulate(float *dst, float v, int overwrite) {
+    *dst = overwrite ? v : *dst + v;
+}
+
 struct BwdCfGeom {
     int32_t streaming;        // aligned rows, whole step pairs: the streaming kernel applies
     int32_t vecs_per_seg;     // multiple of 64
@@ -289,8 +294,8 @@ bwd_channelfirst_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__res
         if (g.n_parts == 1) {
 #pragma unroll
             for (int w = 0; w < W; ++w)
-                p.dweight[(int64_t)c * p.dw_stride_c + (int64_t)w * p.dw_stride_w] += dW[w];
-            if (p.dbias != nullptr) p.dbias[c] += dB;
+                accumulate(p.dweight + (int64_t)c * p.dw_stride_c + (int64_t)w * p.dw_stride_w, dW[w], p.overwrite_dweight);
+            if (p.dbias != nullptr) accumulate(p.dbias + c, dB, p.overwrite_dweight);
         } else {
             float *dst = ws + (int64_t)part * (W + 1) * p.dim + c;
 #pragma unroll
@@ -511,8 +516,8 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
         if (g.n_parts == 1) {
 #pragma unroll
             for (int w = 0; w < W; ++w)
-                p.dweight[(int64_t)c * p.dw_stride_c + (int64_t)w * p.dw_stride_w] += dW[w];
-            if (p.dbias != nullptr) p.dbias[c] += dB;
+                accumulate(p.dweight + (int64_t)c * p.dw_stride_c + (int64_t)w * p.dw_stride_w, dW[w], p.overwrite_dweight);
+            if (p.dbias != nullptr) accumulate(p.dbias + c, dB, p.overwrite_dweight);
         } else {
             float *dst = ws + (int64_t)part * (W + 1) * p.dim + c;
 #pragma unroll

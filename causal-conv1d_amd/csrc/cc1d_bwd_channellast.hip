@@ -19,8 +19,10 @@
 // uniform: two loads, one store and the same arithmetic for every row, no branch.  The last
 // run of a sequence adds the W-1 closing rows, run 0 routes rows in front of the sequence
 // to dinitial_states.  A lane's dweight/dbias partial sums stay in registers for the whole
-// run (no cross-lane reduction, no atomics); each run stores them to a workspace plane and
-// a second kernel adds the planes up in a fixed order: results are bit-reproducible.
+// run (no cross-lane reduction, no atomics).  The four wavefronts of a workgroup take four
+// consecutive runs of the same columns; their partial sums are added through LDS in the order
+// of the runs and stored as one workspace plane, and a second kernel adds the planes up in a
+// fixed order: results are bit-reproducible.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -40,41 +42,32 @@ namespace {
 
 constexpr int kXcds = 8;
 
+constexpr int kRunsPerBlock = kBlock / kWave;   // the wavefronts of a workgroup take consecutive runs
+
 struct BwdClGeom {
     int32_t rows_per_run;     // T, a multiple of twice the unroll factor
     int32_t n_runs;           // ceil(seqlen / T)
+    int32_t n_quads;          // ceil(n_runs / 4): workgroups along one sequence
     int32_t n_colgroups;      // dim / CH
-    uint32_t waves_per_row;   // ceil(n_colgroups / 64): wavefronts side by side on one row
-    uint32_t total;           // batch * n_runs * waves_per_row wavefronts
+    uint32_t waves_per_row;   // ceil(n_colgroups / 64): workgroups side by side on one row
+    uint32_t total;           // batch * n_quads * waves_per_row workgroups
     uint32_t blocks_per_xcd;  // grid size / 8
     int32_t w_fast;           // weights_contiguous_f32
     int32_t w_mode;           // weights_mode: 0 general loader, 1 / 2 packed taps
 };
 
-// WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
-// through PackedTaps), 0: any layout and type (general loader).
+// One wavefront's walk over run `run` of sequence b, columns col*CH .. col*CH+CH per lane: writes
+// dx (and dinitial_states) and returns the lane's dweight / dbias terms in dW / dB.
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
-__global__ void __launch_bounds__(kBlock, CC1D_BWD_CL_OCC)
-bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws,
-                       const int32_t *__restrict__ seq_idx) {
+__device__ __forceinline__ void
+bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t *__restrict__ seq_idx,
+                    const int b, const int run, const uint32_t col, float (&dW)[CH][W], float (&dB)[CH]) {
     using E = Elem<DT>;
     using T_ = typename E::type;
     using P = Pack<DT, CH>;
     using raw_t = typename P::raw_t;
     constexpr bool PRECISE = E::kPreciseAct;
 
-    // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
-    const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
-    // A wavefront takes 64 adjacent vector-columns of one (batch, run): its row range and
-    // the sub-sequence ids it reads are scalars.
-    const uint32_t wave = block * (uint32_t)(kBlock / kWave) +
-                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
-    if (wave >= g.total) return;
-    const uint32_t col = (wave % g.waves_per_row) * (uint32_t)kWave + (threadIdx.x & (kWave - 1));
-    const uint32_t rb = wave / g.waves_per_row;
-    if (col >= (uint32_t)g.n_colgroups) return;       // no cross-lane traffic below
-    const int run = (int)(rb % (uint32_t)g.n_runs);
-    const int b = (int)(rb / (uint32_t)g.n_runs);
     const int c0 = (int)col * CH;
     const int L = p.seqlen;
     const int T = g.rows_per_run;
@@ -222,14 +215,6 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
         mixed = lo != hi || (int)hi < 0;
     }
 
-    float dW[CH][W], dB[CH];
-#pragma unroll
-    for (int j = 0; j < CH; ++j) {
-        dB[j] = 0.f;
-#pragma unroll
-        for (int w = 0; w < W; ++w) dW[j][w] = 0.f;
-    }
-
     // CHECKED = false: loads and stores are unconditional (the wait counts the compiler
     // derives are then exact and loads stay in flight across stores).  CHECKED = true: the
     // first rows of run 0 (positions in front of the sequence go to dinitial_states) and
@@ -374,21 +359,72 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
         }
     }
 
-    // Partials of this run: plane w of part (b, run), channels c0 .. c0+CH.
-    const int64_t part = (int64_t)b * g.n_runs + run;
-    float *dst = ws + part * (int64_t)(W + 1) * p.dim + c0;
+}
+
+// WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
+// through PackedTaps), 0: any layout and type (general loader).
+template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
+__global__ void __launch_bounds__(kBlock, CC1D_BWD_CL_OCC)
+bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws,
+                       const int32_t *__restrict__ seq_idx) {
+    // Partial sums of wavefronts 1..3, one float per lane and term.
+    __shared__ float partial[kRunsPerBlock - 1][(W + 1) * CH][kWave];
+
+    // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
+    const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
+    // A workgroup takes 64 adjacent vector-columns of four consecutive runs of one sequence,
+    // one run per wavefront: a wavefront's row range and the sub-sequence ids it reads are
+    // scalars.  Neighbouring workgroups take neighbouring columns of the same rows.
+    const int wv_in_block = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const int lane = (int)(threadIdx.x & (kWave - 1));
+    const uint32_t col = (block % g.waves_per_row) * (uint32_t)kWave + (uint32_t)lane;
+    const uint32_t bq = block / g.waves_per_row;
+    const int quad = (int)(bq % (uint32_t)g.n_quads);
+    const int b = (int)(bq / (uint32_t)g.n_quads);
+    const int run = quad * kRunsPerBlock + wv_in_block;
+
+    float dW[CH][W], dB[CH];
 #pragma unroll
-    for (int w = 0; w <= W; ++w) {
-        typename RawBytes<CH * 4>::type o;
+    for (int j = 0; j < CH; ++j) {
+        dB[j] = 0.f;
 #pragma unroll
-        for (int j = 0; j < CH; ++j) o[j] = bitcast<uint32_t>(w < W ? dW[j][w] : dB[j]);
-        *reinterpret_cast<typename RawBytes<CH * 4>::type *>(dst + (int64_t)w * p.dim) = o;
+        for (int w = 0; w < W; ++w) dW[j][w] = 0.f;
+    }
+    // Workgroups past the end of the grid's last XCD slice, runs past the end of the sequence
+    // and lanes past the last column have nothing to walk; they still meet the barrier below.
+    const bool active = block < g.total && run < g.n_runs && col < (uint32_t)g.n_colgroups;
+    if (active) bwd_channellast_run<DT, CH, W, HAS_SEQ, SILU, U, WM>(p, g, seq_idx, b, run, col, dW, dB);
+
+    // The workgroup's four partial sums are added in the order of the runs and stored once:
+    // plane w of part (b, quad), channels c0 .. c0+CH.
+    if (wv_in_block > 0) {
+#pragma unroll
+        for (int w = 0; w <= W; ++w)
+#pragma unroll
+            for (int j = 0; j < CH; ++j) partial[wv_in_block - 1][w * CH + j][lane] = w < W ? dW[j][w] : dB[j];
+    }
+    __syncthreads();
+    if (wv_in_block == 0 && block < g.total && col < (uint32_t)g.n_colgroups) {
+        const int64_t part = (int64_t)b * g.n_quads + quad;
+        float *dst = ws + part * (int64_t)(W + 1) * p.dim + (int64_t)col * CH;
+#pragma unroll
+        for (int w = 0; w <= W; ++w) {
+            typename RawBytes<CH * 4>::type o;
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                float v = w < W ? dW[j][w] : dB[j];
+#pragma unroll
+                for (int r = 0; r < kRunsPerBlock - 1; ++r) v += partial[r][w * CH + j][lane];
+                o[j] = bitcast<uint32_t>(v);
+            }
+            *reinterpret_cast<typename RawBytes<CH * 4>::type *>(dst + (int64_t)w * p.dim) = o;
+        }
     }
 }
 
 }  // namespace
 
-// Second stage shared by both backward layouts: dweight[c, w] += sum over parts of
+// Second stage shared by both backward layouts: dweight[c, w] += (or =) sum over parts of
 // ws[part][w][c]; plane W holds dbias.  A workgroup owns 64 channels of one plane; its 16
 // wavefronts each add up every 16th part (four independent chains, so the loads overlap),
 // and wavefront 0 combines the 16 slice sums through LDS.  The order of the additions is a
@@ -399,7 +435,7 @@ constexpr int kFinChannels = 64;
 __global__ void __launch_bounds__(kFinSlices * kFinChannels)
 bwd_finalize_kernel(const float *__restrict__ ws, int n_parts, int dim, int width,
                     float *__restrict__ dweight, int64_t dw_stride_c, int64_t dw_stride_w,
-                    float *__restrict__ dbias) {
+                    float *__restrict__ dbias, int overwrite) {
     __shared__ float slice_sum[kFinSlices][kFinChannels];
     const int lane = (int)threadIdx.x % kFinChannels;
     const int slice = (int)threadIdx.x / kFinChannels;
@@ -427,8 +463,8 @@ bwd_finalize_kernel(const float *__restrict__ ws, int n_parts, int dim, int widt
         float total = 0.f;
 #pragma unroll
         for (int i = 0; i < kFinSlices; ++i) total += slice_sum[i][lane];
-        if (w < width) dweight[(int64_t)c * dw_stride_c + (int64_t)w * dw_stride_w] += total;
-        else dbias[c] += total;
+        float *dst = w < width ? dweight + (int64_t)c * dw_stride_c + (int64_t)w * dw_stride_w : dbias + c;
+        *dst = overwrite ? total : *dst + total;
     }
 }
 
@@ -436,7 +472,8 @@ int launch_bwd_finalize(const float *ws, int n_parts, const cc1d_bwd_params &p, 
     const uint32_t planes = (uint32_t)p.width + (p.dbias != nullptr ? 1u : 0u);
     const uint32_t cblocks = ((uint32_t)p.dim + kFinChannels - 1) / kFinChannels;
     hipLaunchKernelGGL(bwd_finalize_kernel, dim3(planes * cblocks), dim3(kFinSlices * kFinChannels), 0, stream,
-                       ws, n_parts, p.dim, p.width, p.dweight, p.dw_stride_c, p.dw_stride_w, p.dbias);
+                       ws, n_parts, p.dim, p.width, p.dweight, p.dw_stride_c, p.dw_stride_w, p.dbias,
+                       p.overwrite_dweight);
     return launch_status();
 }
 
@@ -449,16 +486,12 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     constexpr int U2 = 2 * CC1D_BWD_CL_UNROLL;        // the walk is unrolled over two groups
     g.n_colgroups = p.dim / channels_per_lane(p.x_dtype);
     int T = tunables().bwd_cl_rows;
-    // Runs of 128 rows: the halo in front of a run and its partial-sum planes then cost about
-    // 5% of the tensor traffic while the prefill shape still launches 2688 wavefronts; measured
-    // best against 32, 64 and 256 there.  With seq_idx 64 rows do better: fewer runs then
-    // contain a sub-sequence boundary and need the masked walk.
-    if (T <= 0) {
-        T = p.seq_idx != nullptr ? 64 : 128;
-        // Small problems: shorter runs until about 8 wavefronts per CU exist.
-        const int64_t target_lanes = (int64_t)256 * 8 * kWave;
-        while (T > 32 && (int64_t)p.batch * g.n_colgroups * ((p.seqlen + T - 1) / T) < target_lanes) T >>= 1;
-    }
+    // Runs of 32 rows, four of them per workgroup: the halo in front of a run costs 9 % more row
+    // requests (found in cache: the run in front belongs to the same workgroup or the one
+    // before), a workgroup's partial sums are one plane per 128 rows, and the prefill shape
+    // launches 10752 wavefronts.  Measured there against 16, 24, 48, 64 and 128 rows, with and
+    // without seq_idx.
+    if (T <= 0) T = 32;
     const int cap = (p.seqlen + U2 - 1) / U2 * U2;     // never longer than the sequence
     if (T > cap) T = cap;
     T = (T + U2 - 1) / U2 * U2;
@@ -470,12 +503,12 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     if ((int64_t)(T + U2) * row_bytes >= ((int64_t)1 << 31)) return false;
     g.rows_per_run = T;
     g.n_runs = (p.seqlen + T - 1) / T;
+    g.n_quads = (g.n_runs + kRunsPerBlock - 1) / kRunsPerBlock;
     g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
-    const int64_t total = (int64_t)p.batch * g.n_runs * g.waves_per_row;
-    if (total * kWave >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
+    const int64_t total = (int64_t)p.batch * g.n_quads * g.waves_per_row;    // workgroups
+    if (total * kBlock >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
     g.total = (uint32_t)total;
-    const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
-    g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
+    g.blocks_per_xcd = (uint32_t)((total + kXcds - 1) / kXcds);
     g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
     g.w_mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     return true;
@@ -516,7 +549,7 @@ int launch_dtype(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStr
 size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p) {
     BwdClGeom g;
     if (!make_geom(p, g)) return 0;
-    return (size_t)p.batch * g.n_runs * (p.width + 1) * (size_t)p.dim * sizeof(float);
+    return (size_t)p.batch * g.n_quads * (p.width + 1) * (size_t)p.dim * sizeof(float);
 }
 
 int launch_bwd_channellast(const cc1d_bwd_params &p, void *workspace, hipStream_t stream) {
@@ -530,7 +563,7 @@ int launch_bwd_channellast(const cc1d_bwd_params &p, void *workspace, hipStream_
         default: st = launch_dtype<CC1D_BF16, 4>(p, g, ws, stream); break;
     }
     if (st != CC1D_OK) return st;
-    return launch_bwd_finalize(ws, p.batch * g.n_runs, p, stream);
+    return launch_bwd_finalize(ws, p.batch * g.n_quads, p, stream);
 }
 
 }  // namespace cc1d

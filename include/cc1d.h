@@ -109,8 +109,9 @@ int cc1d_fwd(const cc1d_fwd_params *p, cc1d_stream_t stream);
  *
  * dweight (fp32, (dim, width)) and dbias (fp32, (dim,)) are ACCUMULATED INTO, like the
  * reference (atomicAdd at bwd.cu:243,255 / add_ at causal_conv1d.cpp:452-459): the
- * caller zeroes them first.  The reduction is always a fixed-order two-stage sum
- * (per-wave partials in the workspace, then one ordered pass), so results are
+ * caller zeroes them first.  With overwrite_dweight = 1 they are plain outputs instead and
+ * need no zeroing (two fill launches fewer per backward call).  The reduction is always a
+ * fixed-order two-stage sum (partials in the workspace, then one ordered pass), so results are
  * bit-reproducible run to run; the reference's `deterministic` switch
  * (causal_conv1d.cpp:21-28, 388-437) has nothing left to select.
  *
@@ -123,7 +124,7 @@ typedef struct cc1d_bwd_params {
     int32_t x_dtype;                 /* of x, dout, dx, initial_states, dfinal_states, dinitial_states */
     int32_t w_dtype;                 /* of weight, bias */
     int32_t silu;
-    int32_t reserved0;
+    int32_t overwrite_dweight;       /* 0: add into dweight / dbias; 1: store the sums, ignore what was there */
 
     const void *x;
     int64_t x_stride_b, x_stride_c, x_stride_l;
@@ -140,9 +141,9 @@ typedef struct cc1d_bwd_params {
 
     void *dx;                        /* same layout family as x */
     int64_t dx_stride_b, dx_stride_c, dx_stride_l;
-    float *dweight;                  /* fp32 (dim, width), accumulated into */
+    float *dweight;                  /* fp32 (dim, width), accumulated into (or overwritten) */
     int64_t dw_stride_c, dw_stride_w;
-    float *dbias;                    /* fp32 (dim,) unit stride, accumulated into, or NULL */
+    float *dbias;                    /* fp32 (dim,) unit stride, like dweight, or NULL */
     void *dinitial_states;           /* or NULL */
     int64_t dinit_stride_b, dinit_stride_c, dinit_stride_l;
 } cc1d_bwd_params;

@@ -27,7 +27,7 @@ class FwdParams(C.Structure):
 class BwdParams(C.Structure):
     _fields_ = [
         ("batch", i32), ("dim", i32), ("seqlen", i32), ("width", i32),
-        ("x_dtype", i32), ("w_dtype", i32), ("silu", i32), ("reserved0", i32),
+        ("x_dtype", i32), ("w_dtype", i32), ("silu", i32), ("overwrite_dweight", i32),
         ("x", vp), ("x_stride_b", i64), ("x_stride_c", i64), ("x_stride_l", i64),
         ("weight", vp), ("w_stride_c", i64), ("w_stride_w", i64),
         ("bias", vp),

@@ -173,6 +173,38 @@ def test_bwd_c_abi_accumulates_into_dweight(gpu_device, cc1d_lib, channel_last):
     assert_close(db + 1.0, ref[2], what="dbias", tol=TOL_W)
 
 
+@pytest.mark.parametrize("channel_last,dim,seqlen", [(False, 64, 500), (False, 4096, 64), (True, 64, 500),
+                                                     (True, 64, 0)])
+def test_bwd_c_abi_overwrite_dweight(gpu_device, cc1d_lib, channel_last, dim, seqlen):
+    """overwrite_dweight = 1: dweight / dbias are plain outputs.  Whatever they held (NaN here)
+    is ignored and the sums equal, bit for bit, the ones accumulated into zeros; an empty
+    problem stores zeros.  dim 4096 channel-first is the path without a second stage."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    g = gen(78)
+    x = make_x(2, dim, seqlen, torch.bfloat16, channel_last, g, sliced=False).to(dev)
+    dout = make_x(2, dim, seqlen, torch.bfloat16, channel_last, g, sliced=False).to(dev)
+    w, b = (t.to(dev) for t in make_wb(dim, 4, True, g))
+    stream = torch.cuda.current_stream().cuda_stream
+    got = []
+    for overwrite, fill in ((0, 0.0), (1, float("nan"))):
+        dx = torch.empty_like(x)
+        dw = torch.full((dim, 4), fill, device=dev)
+        db = torch.full((dim,), fill, device=dev)
+        p = cabi.bwd_params(x, w, b, dout, dx, dw, db, True)
+        p.overwrite_dweight = overwrite
+        need = ctypes.c_size_t()
+        assert lib.cc1d_bwd_workspace_bytes(ctypes.byref(p), ctypes.byref(need)) == 0
+        ws = torch.empty(max(16, need.value), dtype=torch.uint8, device=dev)
+        st = lib.cc1d_bwd(ctypes.byref(p), ws.data_ptr(), need.value, stream)
+        assert st == 0, lib.cc1d_strerror(st)
+        torch.cuda.synchronize()
+        got.append((dw, db))
+    assert torch.equal(got[0][0], got[1][0]) and torch.equal(got[0][1], got[1][1])
+    if seqlen == 0:
+        assert not got[1][0].any() and not got[1][1].any()
+
+
 def test_bwd_full_size_fp16_channel_first_with_states(pkg, gpu_device):
     """The backward configuration at full size: fp16 (4, 4096, 8192) channel-first, width 4,
     SiLU, initial_states and a gradient on final_states.  Channels are independent, so a

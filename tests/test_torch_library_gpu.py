@@ -47,6 +47,10 @@ def test_opcheck_bwd(pkg, gpu_device):
     dinit = torch.empty(2, 3, 256, dtype=x.dtype, device=gpu_device).transpose(1, 2)
     op = torch.ops.DaoAILab._causal_conv1d_bwd_cpp
     torch.library.opcheck(op, (x, w, b, dout, None, init, dfin, dx, dw, db, dinit, True), test_utils=OPCHECKS)
+    # the variant the autograd function uses: dweight / dbias stored, not added to
+    op = torch.ops.DaoAILab._causal_conv1d_bwd_overwrite_cpp
+    torch.library.opcheck(op, (x, w, b, dout, None, init, dfin, dx, torch.empty_like(dw), torch.empty_like(db),
+                               dinit, True), test_utils=OPCHECKS)
 
 
 def test_opcheck_update(pkg, gpu_device):
