@@ -216,6 +216,19 @@ def bench_others(ext, dev, steps, warmup):
                                    "rotated_sets": len(sets), "us_wall_per_call": round(wall, 2)})
         del sets, outs
 
+    # What this box charges for any launch of the decode step's size, measured the same way:
+    # a device-to-device copy moving as many bytes as the linear step (half read, half written)
+    # and a one-element fill (a launch that moves nothing).
+    half = res["update_linear_s3"]["algorithmic_bytes"] // 2
+    src = torch.empty(half, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    one = torch.empty(1, device=dev)
+    us_copy, _ = time_gpu(lambda i: dst.copy_(src), 4 * steps, warmup)
+    us_fill, _ = time_gpu(lambda i: one.fill_(1.0), 4 * steps, warmup)
+    res["launch_floors"] = {"copy_of_update_linear_bytes_us": round(us_copy, 3),
+                            "one_element_fill_us": round(us_fill, 3), "copy_bytes": 2 * half}
+    del src, dst
+
     # C4: backward, fp16 channel-first with initial states and dfinal.
     cfg = to_dev(config_c4(), dev)
     x = cfg["x"]
