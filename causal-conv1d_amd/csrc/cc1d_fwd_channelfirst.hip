@@ -16,12 +16,14 @@
 // initial_states / final_states are supported (the reference refuses them for this
 // layout, csrc/causal_conv1d.cpp:213,228).
 //
-// Two kernels share this design.  The streaming kernel takes rows of x and out that are
-// 16-byte aligned and a whole number of vectors long (seqlen a multiple of 8, or 4 for
-// fp32): whole 64-vector steps run without bounds checks in two register sets in ping-pong,
-// which keep the loads of the next two groups in flight while a group is computed and stored;
-// what is left over at the end of a segment (an odd group, a partly filled step) takes a
-// checked step.  The general kernel takes rows that start off the 16-byte grid.
+// Two kernels share this design.  The streaming kernel takes every launch in which the rows
+// of out lie on the same 16-byte grid as the rows of x (same shape and strides, as
+// empty_like gives): whole 64-vector steps run without bounds checks in two register sets in
+// ping-pong, which keep the loads of the next two groups in flight while a group is computed
+// and stored; what is left over at the end of a segment (fewer than a pair of groups, a partly
+// filled step) is requested at once and then worked off step by step, and the few positions of
+// a row in front of its first whole vector or behind its last one are produced one per lane,
+// straight from memory.  The general kernel takes out tensors on a different grid.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -185,32 +187,59 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
     const T *xr = reinterpret_cast<const T *>(p.x) + xrow;
     T *orow = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b + (int64_t)c * p.out_stride_c;
 
-    const int n_vecs = L / VEC;
-    const int j_begin = seg * g.vecs_per_seg;
+    // The row on its own 16-byte grid (x and out share it): vector j holds positions
+    // j*VEC - mis .. j*VEC - mis + VEC.  Vectors jf0 .. jf1 lie inside the row and move as
+    // vectors; the up to VEC-1 positions in front of them and behind them are edge positions,
+    // each produced by one lane straight from memory.
+    const int mis = (int)((reinterpret_cast<uintptr_t>(xr) / sizeof(T)) % VEC);
+    const int jf0 = mis > 0 ? 1 : 0;
+    const int jf1 = (L + mis) / VEC;
+    int j_begin = seg * g.vecs_per_seg;
     int j_end = j_begin + g.vecs_per_seg;
-    if (j_end > n_vecs) j_end = n_vecs;
-    const int n_groups = (j_end - j_begin) / (2 * kWave * U) * 2;   // whole groups of U steps, in pairs
+    const bool owns_tail = j_begin <= jf1 && jf1 < j_end;
+    if (j_begin < jf0) j_begin = jf0;
+    if (j_end > jf1) j_end = jf1;
+    // whole groups of U steps, in pairs
+    const int n_groups = j_begin < j_end ? (j_end - j_begin) / (2 * kWave * U) * 2 : 0;
+
+    float wv[W], bias_v;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+        wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
+    bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+    if (SCALED) {
+        bias_v *= kSiluPrescale;
+#pragma unroll
+        for (int w = 0; w < W; ++w) wv[w] *= kSiluPrescale;
+    }
+
+    // Edge positions: [0, front) by lanes 0.. of the row's first wave, [back, L) by lanes VEC..
+    // of the wave whose range holds vector jf1.  A row shorter than its first vector is all
+    // front edge.
+    {
+        const int front = mis == 0 ? 0 : (jf1 < jf0 ? L : VEC - mis);
+        const int back = jf1 < jf0 ? L : jf1 * VEC - mis;
+        int t = -1;
+        if (seg == 0 && lane < front) t = lane;
+        if (owns_tail && lane >= VEC && lane - VEC < L - back) t = back + lane - VEC;
+        if (t >= 0) {
+            float a = bias_v;
+#pragma unroll
+            for (int w = 0; w < W; ++w) a = fmaf(wv[w], padded_elem<DT, W>(p, xrow, b, c, t - (W - 1) + w), a);
+            a = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
+            orow[t] = E::from_float(a);
+        }
+    }
 
     if (j_begin < j_end) {
-        float wv[W], bias_v;
-#pragma unroll
-        for (int w = 0; w < W; ++w)
-            wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
-        bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
-        if (SCALED) {
-            bias_v *= kSiluPrescale;
-#pragma unroll
-            for (int w = 0; w < W; ++w) wv[w] *= kSiluPrescale;
-        }
-
         // Halo of the segment's first vector, wave-uniform.
         float carry[W - 1];
 #pragma unroll
         for (int i = 0; i < W - 1; ++i)
-            carry[i] = padded_elem<DT, W>(p, xrow, b, c, j_begin * VEC - (W - 1) + i);
+            carry[i] = padded_elem<DT, W>(p, xrow, b, c, j_begin * VEC - mis - (W - 1) + i);
 
-        const T *xs = xr + (j_begin + lane) * VEC;    // this lane's vector of step 0
-        T *os = orow + (j_begin + lane) * VEC;
+        const T *xs = xr - mis + (j_begin + lane) * VEC;    // this lane's vector of step 0
+        T *os = orow - mis + (j_begin + lane) * VEC;
         auto load_group = [&](int k, u32x4 (&raw)[U]) {
 #pragma unroll
             for (int u = 0; u < U; ++u)
@@ -269,15 +298,23 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
                 compute_group(k + 1, rb);
             }
         }
-        // Steps the pairs did not cover, the last of them possibly partly filled: lanes past
-        // the segment's end read zeros and store nothing.
-        for (int j0 = j_begin + n_groups * U * kWave; j0 < j_end; j0 += kWave) {
-            const bool mine = j0 + lane < j_end;
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            const int s = (j0 - j_begin) / kWave;
-            if (mine) raw = *reinterpret_cast<const u32x4 *>(xs + s * (kWave * VEC));
+        // Steps the pairs did not cover (fewer than 2 U whole ones and possibly a partly filled
+        // one): all requested first, lanes past the segment's end read zeros and store nothing.
+        constexpr int kTail = 2 * U;
+        const int s0 = n_groups * U;                  // first step of the tail
+        u32x4 tail[kTail];
+#pragma unroll
+        for (int q = 0; q < kTail; ++q) {
+            tail[q] = u32x4{0u, 0u, 0u, 0u};
+            if (j_begin + (s0 + q) * kWave + lane < j_end)
+                tail[q] = *reinterpret_cast<const u32x4 *>(xs + (s0 + q) * (kWave * VEC));
+        }
+#pragma unroll
+        for (int q = 0; q < kTail; ++q) {
+            if (j_begin + (s0 + q) * kWave >= j_end) break;
+            const bool mine = j_begin + (s0 + q) * kWave + lane < j_end;
             float xf[VEC];
-            E::unpack(raw, xf);
+            E::unpack(tail[q], xf);
             float xx[VEC + W - 1];
 #pragma unroll
             for (int i = 0; i < W - 1; ++i) {
@@ -294,15 +331,23 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
                 for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
                 acc[e] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
             }
-            if (mine) *reinterpret_cast<u32x4 *>(os + s * (kWave * VEC)) = E::pack(acc);
+            if (mine) *reinterpret_cast<u32x4 *>(os + (s0 + q) * (kWave * VEC)) = E::pack(acc);
         }
     }
 
     // final_states[b, c, i] = xpad[L-(W-1)+i], bit-exact copies, by the row's first wave.
     if (p.final_states != nullptr && seg == 0 && lane < W - 1) {
-        const int t = L - (W - 1) + lane;             // >= 0: a streaming row holds at least one vector
+        const int t = L - (W - 1) + lane;
+        T v = T(0.f);
+        if (t >= 0) {
+            v = ld_raw<DT>(p.x, xrow + t);
+        } else if (p.initial_states != nullptr) {
+            v = ld_raw<DT>(p.initial_states, (int64_t)b * p.init_stride_b +
+                                                 (int64_t)c * p.init_stride_c +
+                                                 (int64_t)(t + W - 1) * p.init_stride_l);
+        }
         st_raw<DT>(p.final_states, (int64_t)b * p.final_stride_b + (int64_t)c * p.final_stride_c +
-                                       (int64_t)lane * p.final_stride_l, ld_raw<DT>(p.x, xrow + t));
+                                       (int64_t)lane * p.final_stride_l, v);
     }
 }
 
@@ -334,13 +379,15 @@ int launch_dtype(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t strea
 
 int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     const int vec = vec_elems(p.x_dtype);
-    const bool aligned = aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
-                         aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
-    // The streaming kernel needs whole vectors (and W-1 <= one vector for final_states);
+    // The streaming kernel needs every row of out on the 16-byte grid of the same row of x;
     // steps per register set: two once a row has at least eight steps.
-    const int streaming = !(aligned && p.seqlen % vec == 0) ? 0 : p.seqlen >= 8 * kWave * vec ? 2 : 1;
+    const int eb = elem_bytes(p.x_dtype);
+    const bool same_grid = (reinterpret_cast<uintptr_t>(p.x) - reinterpret_cast<uintptr_t>(p.out)) % 16 == 0 &&
+                           reinterpret_cast<uintptr_t>(p.x) % eb == 0 &&
+                           (p.x_stride_b - p.out_stride_b) % vec == 0 && (p.x_stride_c - p.out_stride_c) % vec == 0;
+    const int streaming = !same_grid ? 0 : p.seqlen >= 8 * kWave * vec ? 2 : 1;
     // Worst case over row alignments: a row may start up to vec-1 elements into its grid.
-    const int64_t max_vecs = streaming ? p.seqlen / vec : ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
+    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
     const int64_t rows = (int64_t)p.batch * p.dim;
     int64_t vps;
     if (tunables().fwd_cf_vecs > 0) {
