@@ -147,7 +147,16 @@ struct StepArgs {
     uint32_t n_colgroups;
 };
 
-// Decode step, one token.  Grid: x = blocks of 256 lanes over dim / CH, y = batch / R.
+// Decode step, one token.  A workgroup takes 64 adjacent column groups (one per lane) of
+// 4 x R batch entries (R per wavefront): grid x = blocks of 64 column groups, y = batch / (4 R).
+// The taps and bias of the 64 column groups are the same for the four wavefronts and make up
+// more bytes per lane than its data, so the workgroup fetches them once, word by word, into
+// LDS (laid out in 8-byte units so that the reads back are free of bank conflicts) instead of
+// each lane loading its own: a quarter of the vector-memory instructions for them.  They are
+// requested first, the lane's data rows right behind, and the LDS round trip happens while the
+// data is in flight.
+constexpr int kStepWaves = kBlock / kWave;
+
 template <int DT, int CH, int W, bool CIRC, bool SILU, int R, int WM>
 __global__ void __launch_bounds__(kBlock)
 update_step_kernel(const StepArgs a) {
@@ -155,15 +164,40 @@ update_step_kernel(const StepArgs a) {
     using T = typename E::type;
     using P = Pack<DT, CH>;
     using raw_t = typename P::raw_t;
+    using Taps = PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)>;
     constexpr bool PRECISE = E::kPreciseAct;
+    constexpr int kTapUnits = Taps::kWords / 2, kBiasUnits = Taps::kBiasWords / 2;
+    static_assert(Taps::kWords % 2 == 0 && Taps::kBiasWords % 2 == 0, "staged in 8-byte units");
+    __shared__ u32x2 staged[kTapUnits + kBiasUnits][kWave];
 
-    const uint32_t col = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
-    if (col >= a.n_colgroups) return;
-    const int c0 = (int)col * CH;
+    const uint32_t lc = threadIdx.x & (kWave - 1);
+    const int wave_row = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const uint32_t col0 = blockIdx.x * (uint32_t)kWave;            // < n_colgroups by the grid's size
+    const uint32_t cols_here = a.n_colgroups - col0 < (uint32_t)kWave ? a.n_colgroups - col0 : (uint32_t)kWave;
+    // Lanes past the last column group shadow the block's first one: every address they form
+    // is valid, and they store nothing.
+    const bool col_ok = lc < cols_here;
+    const int c0 = (int)(col0 + (col_ok ? lc : 0u)) * CH;
     const int S = a.state_len;
     const T *xb = reinterpret_cast<const T *>(a.x);
     T *ob = reinterpret_cast<T *>(a.out);
     T *sbase = reinterpret_cast<T *>(a.conv_state);
+
+    // The workgroup's taps, one 32-bit word per thread and trip.
+    constexpr int kElem = Taps::k32 ? 4 : 2;
+    constexpr int kTapTrips = (kWave * Taps::kWords + kBlock - 1) / kBlock;
+    const uint32_t *wsrc = reinterpret_cast<const uint32_t *>(
+        reinterpret_cast<const char *>(a.weight) + (int64_t)col0 * (CH * W * kElem));
+    uint32_t tap_word[kTapTrips], bias_word = 0u;
+#pragma unroll
+    for (int q = 0; q < kTapTrips; ++q) {
+        const uint32_t wi = (uint32_t)q * kBlock + threadIdx.x;
+        tap_word[q] = wi < cols_here * (uint32_t)Taps::kWords ? wsrc[wi] : 0u;
+    }
+    static_assert(kWave * Taps::kBiasWords <= kBlock, "one trip for the bias");
+    if (a.bias != nullptr && threadIdx.x < cols_here * (uint32_t)Taps::kBiasWords)
+        bias_word = reinterpret_cast<const uint32_t *>(
+            reinterpret_cast<const char *>(a.bias) + (int64_t)col0 * (CH * kElem))[threadIdx.x];
 
     // Everything this lane reads is requested up front.
     raw_t rw[R][W - 1], xr[R];
@@ -172,7 +206,7 @@ update_step_kernel(const StepArgs a) {
     bool live[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int b = (int)blockIdx.y * R + r;
+        const int b = ((int)blockIdx.y * kStepWaves + wave_row) * R + r;
         live[r] = b < a.batch;
         const int bb = live[r] ? b : 0;
         const int srow = a.conv_state_indices == nullptr ? bb : a.conv_state_indices[bb];
@@ -188,14 +222,41 @@ update_step_kernel(const StepArgs a) {
         }
         xr[r] = *reinterpret_cast<const raw_t *>(xb + (int64_t)bb * a.x_stride_b + c0);
     }
-    PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
-    taps.request(a.weight, a.bias, c0);
+
+    // Word i of column group g goes to unit i/2 of lane g.
+    {
+        uint32_t *flat = reinterpret_cast<uint32_t *>(&staged[0][0]);
+#pragma unroll
+        for (int q = 0; q < kTapTrips; ++q) {
+            const uint32_t wi = (uint32_t)q * kBlock + threadIdx.x;
+            const uint32_t g = wi / Taps::kWords, i = wi % Taps::kWords;
+            if (wi < (uint32_t)(kWave * Taps::kWords)) flat[((i / 2) * kWave + g) * 2 + (i % 2)] = tap_word[q];
+        }
+        const uint32_t g = threadIdx.x / Taps::kBiasWords, i = threadIdx.x % Taps::kBiasWords;
+        if (threadIdx.x < (uint32_t)(kWave * Taps::kBiasWords))
+            flat[((kTapUnits + i / 2) * kWave + g) * 2 + (i % 2)] = bias_word;
+    }
+    __syncthreads();
+    Taps taps;
+#pragma unroll
+    for (int u = 0; u < kTapUnits; ++u) {
+        const u32x2 v = staged[u][lc];
+        taps.wraw[2 * u] = v.x;
+        taps.wraw[2 * u + 1] = v.y;
+    }
+#pragma unroll
+    for (int u = 0; u < kBiasUnits; ++u) {
+        const u32x2 v = staged[kTapUnits + u][lc];
+        taps.braw[2 * u] = v.x;
+        taps.braw[2 * u + 1] = v.y;
+    }
     float wv[CH][W], bv[CH];
     taps.finish(a.bias != nullptr, wv, bv);
+    if (!col_ok) return;
 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int b = (int)blockIdx.y * R + r;
+        const int b = ((int)blockIdx.y * kStepWaves + wave_row) * R + r;
         if (b >= a.batch) continue;
         raw_t *orow = reinterpret_cast<raw_t *>(ob + (int64_t)b * a.out_stride_b + c0);
         if (!live[r]) {                               // padding slot: zeros out, state untouched
@@ -453,7 +514,8 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         a.state_stride_b = p.state_stride_b; a.state_stride_l = p.state_stride_l;
         a.batch = p.batch; a.state_len = p.state_len;
         a.n_colgroups = (uint32_t)(p.dim / CH);
-        const dim3 grid((a.n_colgroups + kBlock - 1) / kBlock, (uint32_t)((p.batch + kStepRows - 1) / kStepRows));
+        const dim3 grid((a.n_colgroups + kWave - 1) / kWave,
+                        (uint32_t)((p.batch + kStepWaves * kStepRows - 1) / (kStepWaves * kStepRows)));
         auto launch = [&](auto wm) {
             constexpr int WM = decltype(wm)::value;
             if (circ) {
