@@ -150,7 +150,7 @@ struct StepArgs {
 // Decode step, one token.  A workgroup takes 64 adjacent column groups (one per lane) of
 // 4 x R batch entries (R per wavefront): grid x = blocks of 64 column groups, y = batch / (4 R).
 // The taps and bias of the 64 column groups are the same for the four wavefronts and make up
-// more bytes per lane than its data, so the workgroup fetches them once, word by word, into
+// more bytes per lane than its data, so the workgroup fetches them once, 16 bytes per thread, into
 // LDS (laid out in 8-byte units so that the reads back are free of bank conflicts) instead of
 // each lane loading its own: a quarter of the vector-memory instructions for them.  They are
 // requested first, the lane's data rows right behind, and the LDS round trip happens while the
@@ -183,21 +183,34 @@ update_step_kernel(const StepArgs a) {
     T *ob = reinterpret_cast<T *>(a.out);
     T *sbase = reinterpret_cast<T *>(a.conv_state);
 
-    // The workgroup's taps, one 32-bit word per thread and trip.
+    // The workgroup's taps: column group g owns units g*kTapUnits .. of 8 bytes, consecutive in
+    // memory.  A thread fetches one 16-byte pair of units per trip (one unit when a column
+    // group has an odd number of them), and one unit of the bias.
     constexpr int kElem = Taps::k32 ? 4 : 2;
-    constexpr int kTapTrips = (kWave * Taps::kWords + kBlock - 1) / kBlock;
-    const uint32_t *wsrc = reinterpret_cast<const uint32_t *>(
-        reinterpret_cast<const char *>(a.weight) + (int64_t)col0 * (CH * W * kElem));
-    uint32_t tap_word[kTapTrips], bias_word = 0u;
+    constexpr bool kPairs = kTapUnits % 2 == 0;
+    constexpr int kPieces = kPairs ? kWave * kTapUnits / 2 : kWave * kTapUnits;   // per workgroup
+    constexpr int kTapTrips = (kPieces + kBlock - 1) / kBlock;
+    static_assert(kWave * kBiasUnits <= kBlock, "one trip for the bias");
+    const char *wsrc = reinterpret_cast<const char *>(a.weight) + (int64_t)col0 * (CH * W * kElem);
+    const char *bsrc = reinterpret_cast<const char *>(a.bias) + (int64_t)col0 * (CH * kElem);
+    u32x4 tap_piece[kTapTrips];
+    u32x2 bias_unit = {0u, 0u};
 #pragma unroll
     for (int q = 0; q < kTapTrips; ++q) {
-        const uint32_t wi = (uint32_t)q * kBlock + threadIdx.x;
-        tap_word[q] = wi < cols_here * (uint32_t)Taps::kWords ? wsrc[wi] : 0u;
+        const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
+        tap_piece[q] = u32x4{0u, 0u, 0u, 0u};
+        if (pi < cols_here * (uint32_t)(kPieces / kWave)) {
+            if constexpr (kPairs) {
+                tap_piece[q] = reinterpret_cast<const u32x4 *>(wsrc)[pi];
+            } else {
+                const u32x2 v = reinterpret_cast<const u32x2 *>(wsrc)[pi];
+                tap_piece[q].x = v.x;
+                tap_piece[q].y = v.y;
+            }
+        }
     }
-    static_assert(kWave * Taps::kBiasWords <= kBlock, "one trip for the bias");
-    if (a.bias != nullptr && threadIdx.x < cols_here * (uint32_t)Taps::kBiasWords)
-        bias_word = reinterpret_cast<const uint32_t *>(
-            reinterpret_cast<const char *>(a.bias) + (int64_t)col0 * (CH * kElem))[threadIdx.x];
+    if (a.bias != nullptr && threadIdx.x < cols_here * (uint32_t)kBiasUnits)
+        bias_unit = reinterpret_cast<const u32x2 *>(bsrc)[threadIdx.x];
 
     // Everything this lane reads is requested up front.
     raw_t rw[R][W - 1], xr[R];
@@ -223,19 +236,19 @@ update_step_kernel(const StepArgs a) {
         xr[r] = *reinterpret_cast<const raw_t *>(xb + (int64_t)bb * a.x_stride_b + c0);
     }
 
-    // Word i of column group g goes to unit i/2 of lane g.
-    {
-        uint32_t *flat = reinterpret_cast<uint32_t *>(&staged[0][0]);
+    // Unit u of column group g goes to staged[u][g].
 #pragma unroll
-        for (int q = 0; q < kTapTrips; ++q) {
-            const uint32_t wi = (uint32_t)q * kBlock + threadIdx.x;
-            const uint32_t g = wi / Taps::kWords, i = wi % Taps::kWords;
-            if (wi < (uint32_t)(kWave * Taps::kWords)) flat[((i / 2) * kWave + g) * 2 + (i % 2)] = tap_word[q];
+    for (int q = 0; q < kTapTrips; ++q) {
+        const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
+        if (pi < (uint32_t)kPieces) {
+            const uint32_t unit = kPairs ? 2 * pi : pi;
+            const uint32_t g = unit / kTapUnits, u = unit % kTapUnits;
+            staged[u][g] = u32x2{tap_piece[q].x, tap_piece[q].y};
+            if constexpr (kPairs) staged[u + 1][g] = u32x2{tap_piece[q].z, tap_piece[q].w};
         }
-        const uint32_t g = threadIdx.x / Taps::kBiasWords, i = threadIdx.x % Taps::kBiasWords;
-        if (threadIdx.x < (uint32_t)(kWave * Taps::kBiasWords))
-            flat[((kTapUnits + i / 2) * kWave + g) * 2 + (i % 2)] = bias_word;
     }
+    if (threadIdx.x < (uint32_t)(kWave * kBiasUnits))
+        staged[kTapUnits + threadIdx.x % kBiasUnits][threadIdx.x / kBiasUnits] = bias_unit;
     __syncthreads();
     Taps taps;
 #pragma unroll
