@@ -4,9 +4,10 @@
 // Three kernels:
 //  * update_step_kernel — the decode step proper: one new token (seqlen 1) and x, out,
 //    conv_state with unit stride along dim.  A lane owns one 8-byte vector of channels of
-//    two consecutive batch entries; all of its loads (window rows, x, taps) are issued
-//    before anything is consumed, and the grid is (column blocks, batch pairs), so no
-//    index division sits in front of the first load.  This shape moves about 22 MB; its
+//    two consecutive batch entries; all of its loads (window rows, x) are issued before
+//    anything is consumed, the taps come through LDS once per workgroup, and the grid is
+//    (column blocks, batch blocks), so no index division sits in front of the first load.
+//    This shape moves about 22 MB; its
 //    run time is within a microsecond of a plain copy of the same footprint, which itself
 //    only costs about 1.6 us more than an empty launch.
 //  * update_vec_kernel — any seqlen, same unit-stride layout (the
