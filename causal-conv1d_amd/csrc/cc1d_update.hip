@@ -148,16 +148,86 @@ struct StepArgs {
     uint32_t n_colgroups;
 };
 
-// Decode step, one token.  A workgroup takes 64 adjacent column groups (one per lane) of
-// 4 x R batch entries (R per wavefront): grid x = blocks of 64 column groups, y = batch / (4 R).
-// The taps and bias of the 64 column groups are the same for the four wavefronts and make up
-// more bytes per lane than its data, so the workgroup fetches them once, 16 bytes per thread, into
-// LDS (laid out in 8-byte units so that the reads back are free of bank conflicts) instead of
-// each lane loading its own: a quarter of the vector-memory instructions for them.  They are
-// requested first, the lane's data rows right behind, and the LDS round trip happens while the
-// data is in flight.
+// Taps and bias of a workgroup's 64 adjacent column groups (one per lane), fetched once by the
+// whole workgroup and handed to the lanes through LDS.  They are the same for every wavefront
+// of the workgroup and make up more bytes per lane than a decode step's data, so this takes a
+// quarter of the vector-memory instructions that per-lane loads of them would.  Column group g
+// owns kTapUnits consecutive 8-byte units in memory; request() has every thread fetch one
+// 16-byte pair of units per trip (one unit when a column group has an odd number of them) and
+// one unit of the bias, publish() parks them as staged[unit][lane] (read back without bank
+// conflicts), and after a barrier collect() gives a lane its own.  Callers issue request()
+// first and their data loads right behind it, so the LDS round trip happens while the data is
+// in flight.
 constexpr int kStepWaves = kBlock / kWave;
 
+template <class Taps, int CH, int W>
+struct WorkgroupTaps {
+    static constexpr int kTapUnits = Taps::kWords / 2, kBiasUnits = Taps::kBiasWords / 2;
+    static constexpr int kUnits = kTapUnits + kBiasUnits;          // rows of the LDS array
+    static constexpr int kElem = Taps::k32 ? 4 : 2;
+    static constexpr bool kPairs = kTapUnits % 2 == 0;
+    static constexpr int kPieces = kPairs ? kWave * kTapUnits / 2 : kWave * kTapUnits;   // per workgroup
+    static constexpr int kTrips = (kPieces + kBlock - 1) / kBlock;
+    static_assert(Taps::kWords % 2 == 0 && Taps::kBiasWords % 2 == 0, "staged in 8-byte units");
+    static_assert(kWave * kBiasUnits <= kBlock, "one trip for the bias");
+    u32x4 piece[kTrips];
+    u32x2 bias_unit;
+
+    // col0: the workgroup's first column group; cols_here: how many of its 64 exist.
+    __device__ __forceinline__ void request(const void *weight, const void *bias, uint32_t col0, uint32_t cols_here) {
+        const char *wsrc = reinterpret_cast<const char *>(weight) + (int64_t)col0 * (CH * W * kElem);
+        const char *bsrc = reinterpret_cast<const char *>(bias) + (int64_t)col0 * (CH * kElem);
+#pragma unroll
+        for (int q = 0; q < kTrips; ++q) {
+            const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
+            piece[q] = u32x4{0u, 0u, 0u, 0u};
+            if (pi < cols_here * (uint32_t)(kPieces / kWave)) {
+                if constexpr (kPairs) {
+                    piece[q] = reinterpret_cast<const u32x4 *>(wsrc)[pi];
+                } else {
+                    const u32x2 v = reinterpret_cast<const u32x2 *>(wsrc)[pi];
+                    piece[q].x = v.x;
+                    piece[q].y = v.y;
+                }
+            }
+        }
+        bias_unit = u32x2{0u, 0u};
+        if (bias != nullptr && threadIdx.x < cols_here * (uint32_t)kBiasUnits)
+            bias_unit = reinterpret_cast<const u32x2 *>(bsrc)[threadIdx.x];
+    }
+    __device__ __forceinline__ void publish(u32x2 (&staged)[kUnits][kWave]) const {
+#pragma unroll
+        for (int q = 0; q < kTrips; ++q) {
+            const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
+            if (pi < (uint32_t)kPieces) {
+                const uint32_t unit = kPairs ? 2 * pi : pi;
+                const uint32_t g = unit / kTapUnits, u = unit % kTapUnits;
+                staged[u][g] = u32x2{piece[q].x, piece[q].y};
+                if constexpr (kPairs) staged[u + 1][g] = u32x2{piece[q].z, piece[q].w};
+            }
+        }
+        if (threadIdx.x < (uint32_t)(kWave * kBiasUnits))
+            staged[kTapUnits + threadIdx.x % kBiasUnits][threadIdx.x / kBiasUnits] = bias_unit;
+    }
+    static __device__ __forceinline__ void collect(const u32x2 (&staged)[kUnits][kWave], uint32_t lane, Taps &taps) {
+#pragma unroll
+        for (int u = 0; u < kTapUnits; ++u) {
+            const u32x2 v = staged[u][lane];
+            taps.wraw[2 * u] = v.x;
+            taps.wraw[2 * u + 1] = v.y;
+        }
+#pragma unroll
+        for (int u = 0; u < kBiasUnits; ++u) {
+            const u32x2 v = staged[kTapUnits + u][lane];
+            taps.braw[2 * u] = v.x;
+            taps.braw[2 * u + 1] = v.y;
+        }
+    }
+};
+
+// Decode step, one token.  A workgroup takes 64 adjacent column groups (one per lane) of
+// 4 x R batch entries (R per wavefront): grid x = blocks of 64 column groups, y = batch / (4 R).
+// The taps come through WorkgroupTaps.
 template <int DT, int CH, int W, bool CIRC, bool SILU, int R, int WM>
 __global__ void __launch_bounds__(kBlock)
 update_step_kernel(const StepArgs a) {
@@ -167,9 +237,8 @@ update_step_kernel(const StepArgs a) {
     using raw_t = typename P::raw_t;
     using Taps = PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)>;
     constexpr bool PRECISE = E::kPreciseAct;
-    constexpr int kTapUnits = Taps::kWords / 2, kBiasUnits = Taps::kBiasWords / 2;
-    static_assert(Taps::kWords % 2 == 0 && Taps::kBiasWords % 2 == 0, "staged in 8-byte units");
-    __shared__ u32x2 staged[kTapUnits + kBiasUnits][kWave];
+    using Staging = WorkgroupTaps<Taps, CH, W>;
+    __shared__ u32x2 staged[Staging::kUnits][kWave];
 
     const uint32_t lc = threadIdx.x & (kWave - 1);
     const int wave_row = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
@@ -184,34 +253,8 @@ update_step_kernel(const StepArgs a) {
     T *ob = reinterpret_cast<T *>(a.out);
     T *sbase = reinterpret_cast<T *>(a.conv_state);
 
-    // The workgroup's taps: column group g owns units g*kTapUnits .. of 8 bytes, consecutive in
-    // memory.  A thread fetches one 16-byte pair of units per trip (one unit when a column
-    // group has an odd number of them), and one unit of the bias.
-    constexpr int kElem = Taps::k32 ? 4 : 2;
-    constexpr bool kPairs = kTapUnits % 2 == 0;
-    constexpr int kPieces = kPairs ? kWave * kTapUnits / 2 : kWave * kTapUnits;   // per workgroup
-    constexpr int kTapTrips = (kPieces + kBlock - 1) / kBlock;
-    static_assert(kWave * kBiasUnits <= kBlock, "one trip for the bias");
-    const char *wsrc = reinterpret_cast<const char *>(a.weight) + (int64_t)col0 * (CH * W * kElem);
-    const char *bsrc = reinterpret_cast<const char *>(a.bias) + (int64_t)col0 * (CH * kElem);
-    u32x4 tap_piece[kTapTrips];
-    u32x2 bias_unit = {0u, 0u};
-#pragma unroll
-    for (int q = 0; q < kTapTrips; ++q) {
-        const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
-        tap_piece[q] = u32x4{0u, 0u, 0u, 0u};
-        if (pi < cols_here * (uint32_t)(kPieces / kWave)) {
-            if constexpr (kPairs) {
-                tap_piece[q] = reinterpret_cast<const u32x4 *>(wsrc)[pi];
-            } else {
-                const u32x2 v = reinterpret_cast<const u32x2 *>(wsrc)[pi];
-                tap_piece[q].x = v.x;
-                tap_piece[q].y = v.y;
-            }
-        }
-    }
-    if (a.bias != nullptr && threadIdx.x < cols_here * (uint32_t)kBiasUnits)
-        bias_unit = reinterpret_cast<const u32x2 *>(bsrc)[threadIdx.x];
+    Staging staging;
+    staging.request(a.weight, a.bias, col0, cols_here);
 
     // Everything this lane reads is requested up front.
     raw_t rw[R][W - 1], xr[R];
@@ -237,33 +280,10 @@ update_step_kernel(const StepArgs a) {
         xr[r] = *reinterpret_cast<const raw_t *>(xb + (int64_t)bb * a.x_stride_b + c0);
     }
 
-    // Unit u of column group g goes to staged[u][g].
-#pragma unroll
-    for (int q = 0; q < kTapTrips; ++q) {
-        const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
-        if (pi < (uint32_t)kPieces) {
-            const uint32_t unit = kPairs ? 2 * pi : pi;
-            const uint32_t g = unit / kTapUnits, u = unit % kTapUnits;
-            staged[u][g] = u32x2{tap_piece[q].x, tap_piece[q].y};
-            if constexpr (kPairs) staged[u + 1][g] = u32x2{tap_piece[q].z, tap_piece[q].w};
-        }
-    }
-    if (threadIdx.x < (uint32_t)(kWave * kBiasUnits))
-        staged[kTapUnits + threadIdx.x % kBiasUnits][threadIdx.x / kBiasUnits] = bias_unit;
+    staging.publish(staged);
     __syncthreads();
     Taps taps;
-#pragma unroll
-    for (int u = 0; u < kTapUnits; ++u) {
-        const u32x2 v = staged[u][lc];
-        taps.wraw[2 * u] = v.x;
-        taps.wraw[2 * u + 1] = v.y;
-    }
-#pragma unroll
-    for (int u = 0; u < kBiasUnits; ++u) {
-        const u32x2 v = staged[kTapUnits + u][lc];
-        taps.braw[2 * u] = v.x;
-        taps.braw[2 * u + 1] = v.y;
-    }
+    Staging::collect(staged, lc, taps);
     float wv[CH][W], bv[CH];
     taps.finish(a.bias != nullptr, wv, bv);
     if (!col_ok) return;
@@ -311,7 +331,9 @@ update_step_kernel(const StepArgs a) {
 
 // A few tokens per call (2 .. kMaxTokens, speculative decoding): one batch row per lane, every
 // x row and the window requested up front under wave-uniform predicates, then the tokens are
-// produced in order from registers.  Grid: x = blocks of 256 lanes over dim / CH, y = batch.
+// produced in order from registers.  A workgroup takes 64 adjacent column groups of 4 batch
+// entries (one per wavefront): grid x = blocks of 64 column groups, y = batch / 4.  The taps
+// come through WorkgroupTaps.
 constexpr int kMaxTokens = 8;
 
 struct TokensArgs {
@@ -328,23 +350,31 @@ update_tokens_kernel(const TokensArgs ta) {
     using P = Pack<DT, CH>;
     using raw_t = typename P::raw_t;
     constexpr bool PRECISE = E::kPreciseAct;
+    using Taps = PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)>;
+    using Staging = WorkgroupTaps<Taps, CH, W>;
+    __shared__ u32x2 staged[Staging::kUnits][kWave];
     const StepArgs &a = ta.s;
 
-    const uint32_t col = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
-    if (col >= a.n_colgroups) return;
-    const int c0 = (int)col * CH;
-    const int b = (int)blockIdx.y;
+    const uint32_t lc = threadIdx.x & (kWave - 1);
+    const uint32_t col0 = blockIdx.x * (uint32_t)kWave;            // < n_colgroups by the grid's size
+    const uint32_t cols_here = a.n_colgroups - col0 < (uint32_t)kWave ? a.n_colgroups - col0 : (uint32_t)kWave;
+    // Lanes past the last column group and wavefronts past the last batch entry shadow valid
+    // ones (every address they form is valid) up to the barrier and store nothing.
+    const bool col_ok = lc < cols_here;
+    const int c0 = (int)(col0 + (col_ok ? lc : 0u)) * CH;
+    const int b_raw = (int)blockIdx.y * kStepWaves + __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const bool b_ok = b_raw < a.batch;
+    const int b = b_ok ? b_raw : 0;
     const int S = a.state_len;
     const int L = ta.seqlen;                          // 2 .. kMaxTokens
     const T *xrow = reinterpret_cast<const T *>(a.x) + (int64_t)b * a.x_stride_b + c0;
     T *orow = reinterpret_cast<T *>(a.out) + (int64_t)b * a.out_stride_b + c0;
 
+    Staging staging;
+    staging.request(a.weight, a.bias, col0, cols_here);
+
     const int srow = a.conv_state_indices == nullptr ? b : a.conv_state_indices[b];
-    if (srow < 0) {                                   // padding slot: zeros out, state untouched
-        for (int i = 0; i < L; ++i) *reinterpret_cast<raw_t *>(orow + (int64_t)i * ta.out_stride_l) = P::zero();
-        return;
-    }
-    T *st = reinterpret_cast<T *>(a.conv_state) + (int64_t)srow * a.state_stride_b + c0;
+    T *st = reinterpret_cast<T *>(a.conv_state) + (int64_t)(srow < 0 ? 0 : srow) * a.state_stride_b + c0;
     int cs = 0;
     if (CIRC) cs = positive_mod(a.cache_seqlens[b], S);
 
@@ -359,8 +389,16 @@ update_tokens_kernel(const TokensArgs ta) {
         xr[i] = P::zero();
         if (i < L) xr[i] = *reinterpret_cast<const raw_t *>(xrow + (int64_t)i * ta.x_stride_l);
     }
-    PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
-    taps.request(a.weight, a.bias, c0);
+
+    staging.publish(staged);
+    __syncthreads();
+    Taps taps;
+    Staging::collect(staged, lc, taps);
+    if (!col_ok || !b_ok) return;
+    if (srow < 0) {                                   // padding slot: zeros out, state untouched
+        for (int i = 0; i < L; ++i) *reinterpret_cast<raw_t *>(orow + (int64_t)i * ta.out_stride_l) = P::zero();
+        return;
+    }
 
     if (CIRC) {
         int wpos = cs;
@@ -560,7 +598,7 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         a.batch = p.batch; a.state_len = p.state_len;
         a.n_colgroups = (uint32_t)(p.dim / CH);
         ta.x_stride_l = p.x_stride_l; ta.out_stride_l = p.out_stride_l; ta.seqlen = p.seqlen;
-        const dim3 grid((a.n_colgroups + kBlock - 1) / kBlock, (uint32_t)p.batch);
+        const dim3 grid((a.n_colgroups + kWave - 1) / kWave, (uint32_t)((p.batch + kStepWaves - 1) / kStepWaves));
         auto launch = [&](auto wm) {
             constexpr int WM = decltype(wm)::value;
             if (circ) {
