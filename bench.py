@@ -302,8 +302,15 @@ def cpu_baseline(cfg_cpu, n_bytes, gpu_out):
     med = sorted(times)[len(times) // 2]
     err = (gpu_out.float() - ref.float()).abs_()
     parity_ok = bool(torch.all(err <= 5e-2 + 1e-2 * ref.float().abs()))      # bf16: rtol 1e-2, atol 5e-2
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), model)
+    except OSError:
+        pass
     return {"value": round(n_bytes / med * 1e-9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "us_per_call": round(med * 1e6, 1),
+            "kind": "port", "us_per_call": round(med * 1e6, 1), "cpu_model": model,
+            "host_cpu_count": os.cpu_count(),
             "gpu_output_matches": parity_ok, "gpu_max_abs_err": float(err.max()),
             "sample": "the full prefill workload (8 x 5376 x 2048 bf16 + seq_idx), median of %d calls "
                       "of the PyTorch F.conv1d oracle after one warm-up" % len(times)}
