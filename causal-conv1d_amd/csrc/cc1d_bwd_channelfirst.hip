@@ -19,13 +19,15 @@
 // Rows of x, dout and dx may sit on different 16-byte grids; lanes follow x's grid and
 // the other tensors use vectors when they share it, elements otherwise.
 //
-// Two kernels share this design.  The streaming kernel takes rows that are 16-byte aligned
-// and a whole number of vectors long (seqlen a multiple of 8, or 4 for fp32): whole 64-vector
-// steps run without bounds checks in two register sets in ping-pong, and lane 0's x halo is a
-// separate small load of its own, so the sets do not depend on each other and the loads of
-// the next two steps stay in flight while a step is computed; an odd step and the partly
-// filled last step of a row are done first, one checked step at a time.  The general kernel
-// takes rows that start off the 16-byte grid.
+// Two kernels share this design.  The streaming kernel takes every launch in which the rows of
+// dout and dx lie on the 16-byte grid of the same rows of x (same shape and strides): whole
+// 64-vector steps run without bounds checks in two register sets in ping-pong, and lane 0's x
+// halo is a separate small load of its own, so the sets do not depend on each other and the
+// loads of the next two steps stay in flight while a step is computed; an odd step and the
+// partly filled last step of a row are done first, one checked step at a time, and the few
+// positions of a row in front of its first whole vector or behind its last one are done one
+// per lane, straight from memory.  The general kernel takes tensors on different grids and
+// rows shorter than two vectors.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -80,6 +82,49 @@ struct RowCtx {
                                                      (int64_t)c * p.init_stride_c +
                                                      (int64_t)(t + W - 1) * p.init_stride_l);
         return 0.f;
+    }
+    // g[t0 .. t0+N) and the padded x in front of and under them, xp[i] = xpad[t0-(W-1)+i], with
+    // every row access issued unconditionally at a clamped index (one memory round trip for
+    // the whole span, no branch between the loads); positions outside [0, L) give g = 0.
+    template <int N>
+    __device__ __forceinline__ void g_span(int t0, float (&gv)[N], float (&xp)[N + W - 1]) const {
+        using T = typename Elem<DT>::type;
+        const int L = p.seqlen;
+        T xraw[N + W - 1], draw[N];
+#pragma unroll
+        for (int i = 0; i < N + W - 1; ++i) {
+            const int q = t0 - (W - 1) + i;
+            xraw[i] = ld_raw<DT>(p.x, xrow + (q < 0 ? 0 : q >= L ? L - 1 : q));
+        }
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            const int q = t0 + k;
+            draw[k] = ld_raw<DT>(p.dout, drow + (q < 0 ? 0 : q >= L ? L - 1 : q));
+        }
+#pragma unroll
+        for (int i = 0; i < N + W - 1; ++i) {
+            const int q = t0 - (W - 1) + i;
+            xp[i] = q >= 0 && q < L ? Elem<DT>::to_float(xraw[i]) : 0.f;
+        }
+        if (p.initial_states != nullptr && t0 < W - 1) {          // only at a row's start
+#pragma unroll
+            for (int i = 0; i < N + W - 1; ++i) {
+                const int q = t0 - (W - 1) + i;
+                if (q < 0 && q >= -(W - 1)) xp[i] = x_at(q);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            const int q = t0 + k;
+            float gk = q >= 0 && q < L ? Elem<DT>::to_float(draw[k]) : 0.f;
+            if (silu_on) {
+                float z = bias_v;
+#pragma unroll
+                for (int w = 0; w < W; ++w) z = fmaf(wv[w], xp[k + w], z);
+                gk *= silu_grad<Elem<DT>::kPreciseAct>(z);
+            }
+            gv[k] = gk;
+        }
     }
     // g[t] recomputed from memory with the same operation order as the vector path.
     __device__ __forceinline__ float g_at(int t) const {
@@ -340,8 +385,6 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
     const int item_begin = part * g.items_per_part;
     int item_end = item_begin + g.items_per_part;
     if (item_end > g.n_items) item_end = g.n_items;
-    const int n_vecs = L / VEC;
-
     using No = std::integral_constant<bool, false>;
     using Yes = std::integral_constant<bool, true>;
 
@@ -355,30 +398,88 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
         const T *dr = reinterpret_cast<const T *>(p.dout) + rc.drow;
         T *dxr = reinterpret_cast<T *>(p.dx) + (int64_t)b * p.dx_stride_b + (int64_t)c * p.dx_stride_c;
 
-        const int j_begin = seg * g.vecs_per_seg;
+        // The row on its own 16-byte grid (x, dout and dx share it): vector j holds positions
+        // j*VEC - mis .. j*VEC - mis + VEC.  Vectors jf0 .. jf1 lie inside the row and are walked
+        // below; the up to VEC-1 positions in front of them and behind them are edge positions,
+        // each done by one lane straight from memory.
+        const int mis = (int)((reinterpret_cast<uintptr_t>(xr) / sizeof(T)) % VEC);
+        const int jf0 = mis > 0 ? 1 : 0;
+        const int jf1 = (L + mis) / VEC;                // >= jf0: the launcher sends rows shorter than 2 VEC elsewhere
+        int j_begin = seg * g.vecs_per_seg;
         int j_end = j_begin + g.vecs_per_seg;
-        if (j_end > n_vecs) j_end = n_vecs;
+        const bool owns_back = j_begin <= jf1 && jf1 < j_end;
+        if (j_begin < jf0) j_begin = jf0;
+        if (j_end > jf1) j_end = jf1;
+
+        float edge_g = 0.f;                               // g at this lane's edge position
+        const int back = jf1 * VEC - mis;                 // edge positions [back, L)
+        {
+            const int front = mis == 0 ? 0 : VEC - mis;   // and [0, front)
+            int t = -1;
+            if (seg == 0 && lane < front) t = lane;
+            if (owns_back && lane >= VEC && lane - VEC < L - back) t = back + lane - VEC;
+            if (t >= 0) {
+                float gt[W], xp[2 * W - 1];
+                rc.template g_span<W>(t, gt, xp);
+                float a = 0.f;
+#pragma unroll
+                for (int k = 0; k < W; ++k) a = fmaf(rc.wv[W - 1 - k], gt[k], a);
+                if (p.dfinal_states != nullptr && t >= L - (W - 1))
+                    a += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b + (int64_t)c * p.dfinal_stride_c +
+                                                          (int64_t)(t - (L - (W - 1))) * p.dfinal_stride_l);
+                dxr[t] = E::from_float(a);
+                edge_g = gt[0];
+                dB += gt[0];
+#pragma unroll
+                for (int w = 0; w < W; ++w) dW[w] = fmaf(gt[0], xp[w], dW[w]);
+            }
+            // dinitial_states[i] = dx at position i-(W-1) < 0, by the wave that owns the row's
+            // start when the first positions are edge positions (else the walk's lowest step
+            // does it from registers).
+            if (mis > 0 && p.dinitial_states != nullptr && seg == 0 && lane >= 2 * VEC && lane < 2 * VEC + W - 1) {
+                const int i = lane - 2 * VEC;
+                float gi[W], xp[2 * W - 1];
+                rc.template g_span<W>(i - (W - 1), gi, xp);
+                float a = 0.f;
+#pragma unroll
+                for (int k = 0; k < W; ++k) a = fmaf(rc.wv[W - 1 - k], gi[k], a);
+                st_elem<DT>(p.dinitial_states, (int64_t)b * p.dinit_stride_b + (int64_t)c * p.dinit_stride_c +
+                                                   (int64_t)i * p.dinit_stride_l, a);
+            }
+        }
         if (j_begin >= j_end) continue;
         // The item's lowest full steps, an even number of them, go through the ping-pong
-        // pipeline; what is above them (an odd full step, a partly filled last step of the
-        // row) is done first, one checked step at a time.
+        // pipeline; what is above them (an odd full step, a partly filled last step) is done
+        // first, one checked step at a time.
         const int n_steps = (j_end - j_begin) / (2 * kWave) * 2;
         const int j_pipe_end = j_begin + n_steps * kWave;
-        const bool row_top = j_end == n_vecs, row_bottom = j_begin == 0;
+        const bool row_top = j_end == jf1, row_bottom = j_begin == jf0;
+        const T *xg = xr - mis, *dg = dr - mis;         // grid origins
+        T *dxg = dxr - mis;
 
-        // g just right of the item: zero past the row's end, else the next segment's first
-        // positions, recomputed from memory.
+        // g just right of the item: the row's back edge (the lanes above have just computed it),
+        // or the next segment's first positions recomputed from memory; zero past the row's end.
         float carry_g[W - 1];
+        if (row_top && owns_back) {
 #pragma unroll
-        for (int i = 0; i < W - 1; ++i) carry_g[i] = row_top ? 0.f : rc.g_at(j_end * VEC + i);
+            for (int i = 0; i < W - 1; ++i) carry_g[i] = back + i < L ? read_lane(edge_g, VEC + i) : 0.f;
+        } else if (j_end * VEC - mis < L) {
+            float xp[2 * (W - 1)];
+            rc.template g_span<W - 1>(j_end * VEC - mis, carry_g, xp);
+        } else {
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) carry_g[i] = 0.f;
+        }
 
         // Step k counts down the pipeline's range: k = 0 is its highest 64 vectors.
         auto load_step = [&](int k, u32x4 &rx, u32x4 &rd, halo_t &rh) {
-            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;   // first element of the step
-            rx = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xr + e0 + lane * VEC));
-            rd = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(dr + e0 + lane * VEC));
-            const int h0 = e0 >= HALO ? e0 - HALO : 0;              // row start: replaced below
-            rh = *reinterpret_cast<const halo_t *>(xr + h0);
+            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;   // the step's first element on the grid
+            rx = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xg + e0 + lane * VEC));
+            rd = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(dg + e0 + lane * VEC));
+            // The HALO elements in front of the step, or (lowest step of the row, where they
+            // may lie in front of the row and are replaced below) the step's own first ones.
+            const int h0 = e0 - mis >= HALO ? e0 - HALO : e0;
+            rh = *reinterpret_cast<const halo_t *>(xg + h0);
         };
         // top / bottom: compiled in for the steps that can be the item's highest / lowest;
         // top_rt / bottom_rt say whether this one is, and is the row's end as well.
@@ -393,7 +494,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             if (decltype(bottom)::value) {
                 if (bottom_rt) {
 #pragma unroll
-                    for (int i = 0; i < W - 1; ++i) carry_x[i] = rc.x_at(i - (W - 1));
+                    for (int i = 0; i < W - 1; ++i) carry_x[i] = rc.x_at(e0 - mis - (W - 1) + i);
                 }
             }
             // xx[i] = xpad at position tf-(W-1)+i
@@ -418,6 +519,9 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
 #pragma unroll
             for (int i = 0; i < W - 1; ++i) {
                 gg[VEC + i] = from_next_lane(gf[i], carry_g[i]);
+                // A partly filled step: its last vector's right neighbour is what follows the
+                // item, not the idle lane behind it.
+                if (decltype(checked)::value) gg[VEC + i] = lane == nvalid - 1 ? carry_g[i] : gg[VEC + i];
                 carry_g[i] = read_lane(gf[i], 0);
             }
             float dxv[VEC];
@@ -429,16 +533,22 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
                 dxv[e] = a;
             }
             if (decltype(top)::value) {
+                // dfinal_states[i] belongs to position L-(W-1)+i: those of them that lie in the
+                // row's last whole vector (the rest are back-edge positions).
                 if (top_rt && p.dfinal_states != nullptr && lane == nvalid - 1) {
+                    const int first = L - (W - 1) - (e0 - mis + lane * VEC);   // element of this vector at i = 0
 #pragma unroll
-                    for (int i = 0; i < W - 1; ++i)
-                        dxv[VEC - (W - 1) + i] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
-                                                                               (int64_t)c * p.dfinal_stride_c +
-                                                                               (int64_t)i * p.dfinal_stride_l);
+                    for (int e = 0; e < VEC; ++e) {
+                        const int i = e - first;
+                        if (i >= 0 && i < W - 1)
+                            dxv[e] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
+                                                                      (int64_t)c * p.dfinal_stride_c +
+                                                                      (int64_t)i * p.dfinal_stride_l);
+                    }
                 }
             }
             if (!decltype(checked)::value || lane < nvalid)
-                __builtin_nontemporal_store(E::pack(dxv), reinterpret_cast<u32x4 *>(dxr + e0 + lane * VEC));
+                __builtin_nontemporal_store(E::pack(dxv), reinterpret_cast<u32x4 *>(dxg + e0 + lane * VEC));
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 dB += gf[e];
@@ -447,7 +557,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             }
             if (decltype(bottom)::value) {
                 // dinitial_states[i] = dx at position i-(W-1) < 0: only g[0 .. i] reach it.
-                if (bottom_rt && p.dinitial_states != nullptr && lane == 0) {
+                if (bottom_rt && mis == 0 && p.dinitial_states != nullptr && lane == 0) {
 #pragma unroll
                     for (int i = 0; i < W - 1; ++i) {
                         float a = 0.f;
@@ -467,10 +577,10 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             const int e0 = js * VEC;
             u32x4 rx = {0u, 0u, 0u, 0u}, rd = {0u, 0u, 0u, 0u};
             if (lane < nvalid) {
-                rx = *reinterpret_cast<const u32x4 *>(xr + e0 + lane * VEC);
-                rd = *reinterpret_cast<const u32x4 *>(dr + e0 + lane * VEC);
+                rx = *reinterpret_cast<const u32x4 *>(xg + e0 + lane * VEC);
+                rd = *reinterpret_cast<const u32x4 *>(dg + e0 + lane * VEC);
             }
-            const halo_t rh = *reinterpret_cast<const halo_t *>(xr + (e0 >= HALO ? e0 - HALO : 0));
+            const halo_t rh = *reinterpret_cast<const halo_t *>(xg + (e0 - mis >= HALO ? e0 - HALO : e0));
             compute_at(Yes{}, Yes{}, Yes{}, row_top && js + nvalid == j_end, row_bottom && js == j_begin, e0, nvalid,
                        rx, rd, rh);
         }
@@ -527,19 +637,22 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
     }
 }
 
-// Rows of one tensor all start on a 16-byte boundary.
-bool rows_aligned(const void *base, int64_t stride_b, int64_t stride_c, int vec) {
-    return aligned16(base) && stride_b % vec == 0 && stride_c % vec == 0;
+// Every row of tensor b lies on the 16-byte grid of the same row of tensor a.
+bool rows_share_grid(const void *a, int64_t a_stride_b, int64_t a_stride_c, const void *b, int64_t b_stride_b,
+                     int64_t b_stride_c, int vec) {
+    return (reinterpret_cast<uintptr_t>(a) - reinterpret_cast<uintptr_t>(b)) % 16 == 0 &&
+           (a_stride_b - b_stride_b) % vec == 0 && (a_stride_c - b_stride_c) % vec == 0;
 }
 
 BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
-    const bool streaming = p.seqlen % vec == 0 &&
-                           rows_aligned(p.x, p.x_stride_b, p.x_stride_c, vec) &&
-                           rows_aligned(p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
-                           rows_aligned(p.dx, p.dx_stride_b, p.dx_stride_c, vec);
+    // The streaming kernel walks x, dout and dx on one grid per row, and wants a row to hold
+    // at least one whole vector wherever it starts on that grid.
+    const bool streaming = p.seqlen >= 2 * vec && reinterpret_cast<uintptr_t>(p.x) % elem_bytes(p.x_dtype) == 0 &&
+                           rows_share_grid(p.x, p.x_stride_b, p.x_stride_c, p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
+                           rows_share_grid(p.x, p.x_stride_b, p.x_stride_c, p.dx, p.dx_stride_b, p.dx_stride_c, vec);
     // Worst case over row alignments: a row may start up to vec-1 elements into its grid.
-    const int64_t max_vecs = streaming ? p.seqlen / vec : ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
+    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
     const int64_t max_steps = (max_vecs + kWave - 1) / kWave;     // 64-vector steps per row
     // About 16 waves on each of 256 CUs when the problem allows it.
     int64_t parts = tunables().bwd_cf_parts > 0 ? tunables().bwd_cf_parts
