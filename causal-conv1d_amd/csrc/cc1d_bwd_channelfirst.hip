@@ -42,7 +42,7 @@ __device__ __forceinline__ void accumulate(float *dst, float v, int overwrite) {
 }
 
 struct BwdCfGeom {
-    int32_t streaming;        // aligned rows, whole step pairs: the streaming kernel applies
+    int32_t streaming;        // 0: general kernel; streaming kernel with rows 1: on the 16-byte grid, 2: anywhere on it
     int32_t vecs_per_seg;     // multiple of 64
     int32_t n_segs;           // segments per row
     int32_t n_items;          // batch * n_segs
@@ -350,7 +350,10 @@ bwd_channelfirst_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__res
     }
 }
 
-template <int DT, int W>
+// GRID: rows may start anywhere on their 16-byte grid and have any length; false: every row
+// starts on the grid and is a whole number of vectors long (no edge positions exist, and the
+// code for them is compiled out).
+template <int DT, int W, bool GRID>
 __global__ void __launch_bounds__(kBlock)
 bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__restrict__ ws) {
     using E = Elem<DT>;
@@ -402,7 +405,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
         // j*VEC - mis .. j*VEC - mis + VEC.  Vectors jf0 .. jf1 lie inside the row and are walked
         // below; the up to VEC-1 positions in front of them and behind them are edge positions,
         // each done by one lane straight from memory.
-        const int mis = (int)((reinterpret_cast<uintptr_t>(xr) / sizeof(T)) % VEC);
+        const int mis = GRID ? (int)((reinterpret_cast<uintptr_t>(xr) / sizeof(T)) % VEC) : 0;
         const int jf0 = mis > 0 ? 1 : 0;
         const int jf1 = (L + mis) / VEC;                // >= jf0: the launcher sends rows shorter than 2 VEC elsewhere
         int j_begin = seg * g.vecs_per_seg;
@@ -411,6 +414,35 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
         if (j_begin < jf0) j_begin = jf0;
         if (j_end > jf1) j_end = jf1;
 
+        // The item's lowest full steps, an even number of them, go through the ping-pong
+        // pipeline; what is above them (an odd full step, a partly filled last step) is done
+        // first, one checked step at a time.
+        const bool has_vecs = j_begin < j_end;
+        const int n_steps = has_vecs ? (j_end - j_begin) / (2 * kWave) * 2 : 0;
+        const int j_pipe_end = j_begin + n_steps * kWave;
+        const bool row_top = j_end == jf1, row_bottom = j_begin == jf0;
+        const T *xg = xr - mis, *dg = dr - mis;         // grid origins
+        T *dxg = dxr - mis;
+
+        // Step k counts down the pipeline's range: k = 0 is its highest 64 vectors.
+        auto load_step = [&](int k, u32x4 &rx, u32x4 &rd, halo_t &rh) {
+            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;   // the step's first element on the grid
+            rx = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xg + e0 + lane * VEC));
+            rd = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(dg + e0 + lane * VEC));
+            // The HALO elements in front of the step, or (lowest step of the row, where they
+            // may lie in front of the row and are replaced below) the step's own first ones.
+            const int h0 = e0 - mis >= HALO ? e0 - HALO : e0;
+            rh = *reinterpret_cast<const halo_t *>(xg + h0);
+        };
+        // With rows off the grid the pipeline's first two steps are requested before the edge
+        // work, so that its memory round trip and theirs overlap.
+        u32x4 ax, ad, bx, bd;
+        halo_t ah, bh;
+        if (GRID && n_steps > 0) {
+            load_step(0, ax, ad, ah);
+            load_step(1, bx, bd, bh);
+        }
+
         float edge_g = 0.f;                               // g at this lane's edge position
         const int back = jf1 * VEC - mis;                 // edge positions [back, L)
         {
@@ -418,7 +450,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             int t = -1;
             if (seg == 0 && lane < front) t = lane;
             if (owns_back && lane >= VEC && lane - VEC < L - back) t = back + lane - VEC;
-            if (t >= 0) {
+            if (GRID && t >= 0) {
                 float gt[W], xp[2 * W - 1];
                 rc.template g_span<W>(t, gt, xp);
                 float a = 0.f;
@@ -436,7 +468,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             // dinitial_states[i] = dx at position i-(W-1) < 0, by the wave that owns the row's
             // start when the first positions are edge positions (else the walk's lowest step
             // does it from registers).
-            if (mis > 0 && p.dinitial_states != nullptr && seg == 0 && lane >= 2 * VEC && lane < 2 * VEC + W - 1) {
+            if (GRID && mis > 0 && p.dinitial_states != nullptr && seg == 0 && lane >= 2 * VEC && lane < 2 * VEC + W - 1) {
                 const int i = lane - 2 * VEC;
                 float gi[W], xp[2 * W - 1];
                 rc.template g_span<W>(i - (W - 1), gi, xp);
@@ -447,20 +479,11 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
                                                    (int64_t)i * p.dinit_stride_l, a);
             }
         }
-        if (j_begin >= j_end) continue;
-        // The item's lowest full steps, an even number of them, go through the ping-pong
-        // pipeline; what is above them (an odd full step, a partly filled last step) is done
-        // first, one checked step at a time.
-        const int n_steps = (j_end - j_begin) / (2 * kWave) * 2;
-        const int j_pipe_end = j_begin + n_steps * kWave;
-        const bool row_top = j_end == jf1, row_bottom = j_begin == jf0;
-        const T *xg = xr - mis, *dg = dr - mis;         // grid origins
-        T *dxg = dxr - mis;
-
+        if (!has_vecs) continue;
         // g just right of the item: the row's back edge (the lanes above have just computed it),
         // or the next segment's first positions recomputed from memory; zero past the row's end.
         float carry_g[W - 1];
-        if (row_top && owns_back) {
+        if (GRID && row_top && owns_back) {
 #pragma unroll
             for (int i = 0; i < W - 1; ++i) carry_g[i] = back + i < L ? read_lane(edge_g, VEC + i) : 0.f;
         } else if (j_end * VEC - mis < L) {
@@ -471,16 +494,6 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             for (int i = 0; i < W - 1; ++i) carry_g[i] = 0.f;
         }
 
-        // Step k counts down the pipeline's range: k = 0 is its highest 64 vectors.
-        auto load_step = [&](int k, u32x4 &rx, u32x4 &rd, halo_t &rh) {
-            const int e0 = (j_begin + (n_steps - 1 - k) * kWave) * VEC;   // the step's first element on the grid
-            rx = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xg + e0 + lane * VEC));
-            rd = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(dg + e0 + lane * VEC));
-            // The HALO elements in front of the step, or (lowest step of the row, where they
-            // may lie in front of the row and are replaced below) the step's own first ones.
-            const int h0 = e0 - mis >= HALO ? e0 - HALO : e0;
-            rh = *reinterpret_cast<const halo_t *>(xg + h0);
-        };
         // top / bottom: compiled in for the steps that can be the item's highest / lowest;
         // top_rt / bottom_rt say whether this one is, and is the row's end as well.
         auto compute_at = [&](auto top, auto bottom, auto checked, bool top_rt, bool bottom_rt, int e0, int nvalid,
@@ -593,10 +606,10 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
 
         // Two register sets in ping-pong; the first and last pair of steps are peeled so the
         // loop is entered in the state its back edge leaves and the wait counts stay exact.
-        u32x4 ax, ad, bx, bd;
-        halo_t ah, bh;
-        load_step(0, ax, ad, ah);
-        load_step(1, bx, bd, bh);
+        if (!GRID) {
+            load_step(0, ax, ad, ah);
+            load_step(1, bx, bd, bh);
+        }
         if (n_steps == 2) {
             compute_step(Yes{}, No{}, 0, ax, ad, ah);
             compute_step(No{}, Yes{}, 1, bx, bd, bh);
@@ -667,7 +680,8 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     int64_t vps = steps_per_seg * kWave;
     n_segs = (max_vecs + vps - 1) / vps;
     BwdCfGeom g;
-    g.streaming = streaming ? 1 : 0;
+    const bool on_grid = aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 && p.seqlen % vec == 0;
+    g.streaming = !streaming ? 0 : on_grid ? 1 : 2;
     g.vecs_per_seg = (int32_t)vps;
     g.n_segs = (int32_t)n_segs;
     g.n_items = (int32_t)(p.batch * n_segs);
@@ -681,11 +695,19 @@ int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStr
     const int64_t waves = (int64_t)p.dim * g.n_parts;
     if (waves >= ((int64_t)1 << 25)) return CC1D_ERR_TOO_LARGE;
     const uint32_t blocks = (uint32_t)((waves + (kBlock / kWave) - 1) / (kBlock / kWave));
-    if (g.streaming) {
+    if (g.streaming == 1) {                           // rows on the grid, whole vectors
         switch (p.width) {
-            case 2: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            case 3: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            default: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 2: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 2, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 3, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 4, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        }
+        return launch_status();
+    }
+    if (g.streaming == 2) {                           // rows anywhere on the grid
+        switch (p.width) {
+            case 2: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 2, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 3, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 4, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         }
         return launch_status();
     }
