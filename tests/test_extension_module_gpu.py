@@ -98,3 +98,35 @@ def test_prefill_then_decode_equals_one_long_forward(pkg, gpu_device):
         o = pkg.causal_conv1d_update(tok, state, wd, bd, activation="silu")
         for i, (t, n) in enumerate(zip(whole, lens)):
             assert torch.equal(o[i], t[0, :, n + step])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seqlen", [37, 300])
+def test_channel_first_outputs_on_another_16_byte_grid(pkg, gpu_device, dtype, seqlen):
+    """Caller-owned out / dx whose rows sit at other offsets inside their 16-byte vectors than the
+    rows of x (a slice of a wider buffer): the channel-first kernels for that case must give
+    what the same-grid kernels give."""
+    import causal_conv1d_cuda as ext
+    dev = gpu_device
+    g = gen(43 + seqlen)
+    B, D, W = 2, 24, 4
+    x = torch.randn(B, D, seqlen, generator=g).to(dtype)
+    dout = torch.randn(B, D, seqlen, generator=g).to(dtype)
+    w, b = make_wb(D, W, True, g)
+    xd, dd, wd, bd = x.to(dev), dout.to(dev), w.to(dev), b.to(dev)
+    wide = torch.full((B, D, seqlen + 5), float("nan"), dtype=dtype, device=dev)
+    out = wide[:, :, 3:3 + seqlen]                 # rows start 3 elements into the buffer's rows
+    ext.causal_conv1d_fwd(xd, wd, bd, None, None, out, None, True)
+    assert_close(out, orc.fwd(x, w, b, activation="silu"), dtype, "out")
+    assert torch.isnan(wide[:, :, :3]).all() and torch.isnan(wide[:, :, 3 + seqlen:]).all()
+
+    wide_dx = torch.full((B, D, seqlen + 5), float("nan"), dtype=dtype, device=dev)
+    dx = wide_dx[:, :, 1:1 + seqlen]
+    dw = torch.zeros(D, W, device=dev)
+    db = torch.zeros(D, device=dev)
+    ext.causal_conv1d_bwd(xd, wd, bd, dd, None, None, None, dx, dw, db, None, True)
+    ref = orc.bwd(x, w, b, dout, activation="silu")
+    assert_close(dx, ref[0], dtype, "dx")
+    assert_close(dw, ref[1], what="dweight", tol=(1e-3, 1e-3))
+    assert_close(db, ref[2], what="dbias", tol=(1e-3, 1e-3))
+    assert torch.isnan(wide_dx[:, :, :1]).all() and torch.isnan(wide_dx[:, :, 1 + seqlen:]).all()
