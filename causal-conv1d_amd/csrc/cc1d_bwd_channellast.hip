@@ -34,7 +34,7 @@
 #endif
 // Workgroups per CU the register budget must allow.
 #ifndef CC1D_BWD_CL_OCC
-#define CC1D_BWD_CL_OCC 2
+#define CC1D_BWD_CL_OCC 4
 #endif
 
 namespace cc1d {
@@ -364,7 +364,7 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
 // WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
 // through PackedTaps), 0: any layout and type (general loader).
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
-__global__ void __launch_bounds__(kBlock, CC1D_BWD_CL_OCC)
+__global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 4 ? CC1D_BWD_CL_OCC : 2))
 bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__restrict__ ws,
                        const int32_t *__restrict__ seq_idx) {
     // Partial sums of wavefronts 1..3, one float per lane and term.
@@ -479,7 +479,14 @@ int launch_bwd_finalize(const float *ws, int n_parts, const cc1d_bwd_params &p, 
 
 namespace {
 
-int channels_per_lane(int x_dtype) { return vec_elems(x_dtype) / 2; }   // 8-byte lanes
+// Channels per lane for 16-bit tensors: 2, i.e. 4-byte lanes.  A lane's windows, taps and
+// partial sums then fit 128 registers and four workgroups share a CU, which is worth more to
+// this VALU-heavy kernel than wider accesses: 92 us against 102 us with 8-byte lanes and two
+// workgroups per CU at (8, 5376, 2048) bf16.  fp32 keeps 2 channels (8 bytes).
+#ifndef CC1D_BWD_CL_CH16
+#define CC1D_BWD_CL_CH16 2
+#endif
+int channels_per_lane(int x_dtype) { return x_dtype == CC1D_F32 ? 2 : CC1D_BWD_CL_CH16; }   // 8-byte lanes
 
 // Returns false when a run cannot be addressed with 32-bit byte offsets.
 bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
@@ -559,8 +566,8 @@ int launch_bwd_channellast(const cc1d_bwd_params &p, void *workspace, hipStream_
     int st;
     switch (p.x_dtype) {
         case CC1D_F32: st = launch_dtype<CC1D_F32, 2>(p, g, ws, stream); break;
-        case CC1D_F16: st = launch_dtype<CC1D_F16, 4>(p, g, ws, stream); break;
-        default: st = launch_dtype<CC1D_BF16, 4>(p, g, ws, stream); break;
+        case CC1D_F16: st = launch_dtype<CC1D_F16, CC1D_BWD_CL_CH16>(p, g, ws, stream); break;
+        default: st = launch_dtype<CC1D_BF16, CC1D_BWD_CL_CH16>(p, g, ws, stream); break;
     }
     if (st != CC1D_OK) return st;
     return launch_bwd_finalize(ws, p.batch * g.n_quads, p, stream);

@@ -127,9 +127,11 @@ template <> struct Elem<CC1D_BF16> {
 // CH channels of one row held by one lane: a 16-byte or an 8-byte register vector.
 // ---------------------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x1 __attribute__((ext_vector_type(1)));
 template <int BYTES> struct RawBytes;
 template <> struct RawBytes<16> { using type = u32x4; };
 template <> struct RawBytes<8> { using type = u32x2; };
+template <> struct RawBytes<4> { using type = u32x1; };
 
 template <int DT, int CH>
 struct Pack {
