@@ -34,6 +34,16 @@
 #ifndef CC1D_FWD_CL_OCC16
 #define CC1D_FWD_CL_OCC16 2
 #endif
+// Channels per lane of the packed-tap kernels for 16-bit tensors: 2, i.e. 4-byte lanes, compiled
+// for five workgroups per CU (<= 96 registers).  More wavefronts per CU overlap the kernel's
+// VALU time with its memory time better than wider accesses do: 56.1 us against 60.1 us with
+// 8-byte lanes and three workgroups per CU at the prefill shape.  fp32 keeps 2 channels (8 bytes).
+#ifndef CC1D_FWD_CL_CH16
+#define CC1D_FWD_CL_CH16 2
+#endif
+#ifndef CC1D_FWD_CL_OCC4
+#define CC1D_FWD_CL_OCC4 5
+#endif
 #ifndef CC1D_FWD_CL_OCC8
 #define CC1D_FWD_CL_OCC8 3
 #endif
@@ -54,9 +64,9 @@ struct FwdClGeom {
 };
 
 // WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
-// through PackedTaps, 8-byte lanes), 0: any layout and type (general loader, 16-byte lanes).
+// through PackedTaps, narrow lanes), 0: any layout and type (general loader, 16-byte lanes).
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
-__global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CC1D_FWD_CL_OCC8))
+__global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CH * Elem<DT>::kBytes == 4 ? CC1D_FWD_CL_OCC4 : CC1D_FWD_CL_OCC8))
 fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t *__restrict__ seq_idx,
                        const VarlenTail tail) {
     using E = Elem<DT>;
@@ -347,13 +357,15 @@ int launch_width(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail 
     }
 }
 
-// 8-byte lanes with packed taps (mode 1 or 2), else 16-byte lanes with the general loader.
+// Narrow lanes (2 channels: 4 bytes of 16-bit data, 8 bytes of fp32) with packed taps (mode 1
+// or 2), else 16-byte lanes with the general loader.
 template <int DT>
 int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail &tail, int mode, hipStream_t stream) {
     constexpr int FULL = Elem<DT>::kVec;
-    if (mode == 1) return launch_width<DT, FULL / 2, 1>(p, g, tail, stream);
+    constexpr int HALF = DT == CC1D_F32 ? FULL / 2 : CC1D_FWD_CL_CH16;
+    if (mode == 1) return launch_width<DT, HALF, 1>(p, g, tail, stream);
     if constexpr (DT != CC1D_F32) {
-        if (mode == 2) return launch_width<DT, FULL / 2, 2>(p, g, tail, stream);
+        if (mode == 2) return launch_width<DT, HALF, 2>(p, g, tail, stream);
     }
     return launch_width<DT, FULL, 0>(p, g, tail, stream);
 }
@@ -380,13 +392,14 @@ static int choose_rows_per_run(int seqlen, int64_t row_bytes) {
 // gather: a varlen final-state gather to run in the same launch (NULL: none).  It must be one
 // the vector gather takes (varlen_vec_ok) on elements as wide as x's.
 int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *gather, hipStream_t stream) {
-    // Channels per lane: an 8-byte vector (4 x 16-bit or 2 x fp32).  Half the registers of a
-    // 16-byte lane, so twice the waves per SIMD to overlap compute with memory; measured
-    // 9% faster at the prefill shape.  fwd_cl_half_vec = -1 selects 16-byte lanes.
+    // Channels per lane: 2 (4 bytes of 16-bit data, 8 bytes of fp32).  A fraction of the registers
+    // of a 16-byte lane, so more waves per SIMD to overlap compute with memory; measured 9 %
+    // (8-byte lanes) and another 7 % (4-byte lanes) faster at the prefill shape.
+    // fwd_cl_half_vec = -1 selects 16-byte lanes.
     const int full = vec_elems(p.x_dtype);
     int mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     if (tunables().fwd_cl_half_vec < 0) mode = 0;
-    const int ch = mode == 0 ? full : full / 2;
+    const int ch = mode == 0 ? full : p.x_dtype == CC1D_F32 ? full / 2 : CC1D_FWD_CL_CH16;
     FwdClGeom g;
     g.n_colgroups = p.dim / ch;
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
