@@ -10,7 +10,7 @@
 // with every tap additionally masked by seq_idx equality when seq_idx is given.
 //
 // Design.  Same geometry as the channel-last forward: a lane owns CH adjacent channels
-// (one 8-byte vector) and walks a run of T rows in ascending order, holding (W-1)-row
+// (one 4- or 8-byte vector) and walks a run of T rows in ascending order, holding (W-1)-row
 // sliding windows of x and g in registers.  The run owns g[t] (hence the dweight/dbias
 // terms) for its rows t in [t0, t1) and emits dx one window late: row t completes
 // dx[t-(W-1)], so the run writes dx[t0-(W-1) .. t1-(W-1)).  Everything a run needs from
@@ -486,7 +486,7 @@ namespace {
 #ifndef CC1D_BWD_CL_CH16
 #define CC1D_BWD_CL_CH16 2
 #endif
-int channels_per_lane(int x_dtype) { return x_dtype == CC1D_F32 ? 2 : CC1D_BWD_CL_CH16; }   // 8-byte lanes
+int channels_per_lane(int x_dtype) { return x_dtype == CC1D_F32 ? 2 : CC1D_BWD_CL_CH16; }
 
 // Returns false when a run cannot be addressed with 32-bit byte offsets.
 bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {

@@ -3,7 +3,7 @@
 // (csrc/causal_conv1d_fwd.cu:205-381 of the reference).
 //
 // Design.  The stencil runs along seqlen, which is the strided axis, so nothing has to
-// be transposed: a lane owns CH adjacent channels (one 8- or 16-byte vector), keeps their
+// be transposed: a lane owns CH adjacent channels (one 4-, 8- or 16-byte vector), keeps their
 // W taps and bias in registers and walks down a run of consecutive rows with a
 // (W-1)-row sliding window held in registers as fp32.  Per row that is one vector load
 // and one vector store per lane, both fully coalesced along dim, no LDS and no barrier.
@@ -14,8 +14,8 @@
 // ceil(dim / (64 CH)) wavefronts, the last one partly idle when dim is not a multiple of
 // 64 CH.  Wavefronts are numbered (batch, run, column block) with the column block
 // fastest, and workgroups are renumbered so that each of the 8 XCDs (hardware hands
-// workgroups to XCDs round-robin) walks a contiguous slice of that order: the run that follows another along seqlen then executes on the same XCD, close
-// in time, and its halo rows are found in that XCD's L2 instead of being fetched from
+// workgroups to XCDs round-robin) walks a contiguous slice of that order: the run that
+// follows another along seqlen then executes on the same XCD, close in time, and its halo rows are found in that XCD's L2 instead of being fetched from
 // HBM twice.  For the same reason the halo rows and the last rows of a run are accessed
 // with the normal cache policy while everything else streams through (non-temporal).
 #include <type_traits>
@@ -30,7 +30,7 @@
 #ifndef CC1D_FWD_CL_UNROLL16
 #define CC1D_FWD_CL_UNROLL16 4
 #endif
-// Workgroups per CU the register budget must allow, for 16- and 8-byte lanes.
+// Workgroups per CU the register budget must allow, for 16-, 8- and 4-byte lanes.
 #ifndef CC1D_FWD_CL_OCC16
 #define CC1D_FWD_CL_OCC16 2
 #endif
