@@ -3,7 +3,7 @@
 // (csrc/causal_conv1d_fwd.cu:205-381 of the reference).
 //
 // Design.  The stencil runs along seqlen, which is the strided axis, so nothing has to
-// be transposed: a lane owns CH adjacent channels (one 4-, 8- or 16-byte vector), keeps their
+// be transposed: a lane owns CH adjacent channels (one 4- or 8-byte vector), keeps their
 // W taps and bias in registers and walks down a run of consecutive rows with a
 // (W-1)-row sliding window held in registers as fp32.  Per row that is one vector load
 // and one vector store per lane, both fully coalesced along dim, no LDS and no barrier.
@@ -26,16 +26,8 @@
 #ifndef CC1D_FWD_CL_UNROLL
 #define CC1D_FWD_CL_UNROLL 8
 #endif
-// The same for 16-byte lanes, whose rows take twice the registers.
-#ifndef CC1D_FWD_CL_UNROLL16
-#define CC1D_FWD_CL_UNROLL16 4
-#endif
-// Workgroups per CU the register budget must allow, for 16-, 8- and 4-byte lanes.
-#ifndef CC1D_FWD_CL_OCC16
-#define CC1D_FWD_CL_OCC16 2
-#endif
-// Channels per lane of the packed-tap kernels for 16-bit tensors: 2, i.e. 4-byte lanes, compiled
-// for five workgroups per CU (<= 96 registers).  More wavefronts per CU overlap the kernel's
+// Channels per lane for 16-bit tensors: 2, i.e. 4-byte lanes, compiled for five workgroups
+// per CU (<= 96 registers; CC1D_FWD_CL_OCC4), against three for the 8-byte lanes of fp32 data.  More wavefronts per CU overlap the kernel's
 // VALU time with its memory time better than wider accesses do: 56.1 us against 60.1 us with
 // 8-byte lanes and three workgroups per CU at the prefill shape.  fp32 keeps 2 channels (8 bytes).
 #ifndef CC1D_FWD_CL_CH16
@@ -64,9 +56,9 @@ struct FwdClGeom {
 };
 
 // WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
-// through PackedTaps, narrow lanes), 0: any layout and type (general loader, 16-byte lanes).
+// through PackedTaps), 0: any layout and type (general loader).
 template <int DT, int CH, int W, bool HAS_SEQ, bool SILU, int U, int WM>
-__global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_OCC16 : CH * Elem<DT>::kBytes == 4 ? CC1D_FWD_CL_OCC4 : CC1D_FWD_CL_OCC8))
+__global__ void __launch_bounds__(kBlock, (CH * Elem<DT>::kBytes == 4 ? CC1D_FWD_CL_OCC4 : CC1D_FWD_CL_OCC8))
 fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t *__restrict__ seq_idx,
                        const VarlenTail tail) {
     using E = Elem<DT>;
@@ -336,7 +328,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
 
 template <int DT, int CH, int W, bool HAS_SEQ, int WM>
 int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail &tail, hipStream_t stream) {
-    constexpr int U = CH * Elem<DT>::kBytes == 16 ? CC1D_FWD_CL_UNROLL16 : CC1D_FWD_CL_UNROLL;
+    constexpr int U = CC1D_FWD_CL_UNROLL;
     const uint32_t blocks = tail.first_block + (tail.total + kBlock - 1) / kBlock;
     if (p.silu)
         hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>),
@@ -357,8 +349,8 @@ int launch_width(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail 
     }
 }
 
-// Narrow lanes (2 channels: 4 bytes of 16-bit data, 8 bytes of fp32) with packed taps (mode 1
-// or 2), else 16-byte lanes with the general loader.
+// 2 channels per lane (4 bytes of 16-bit data, 8 bytes of fp32); taps through PackedTaps when
+// they are packed (mode 1 or 2), else through the general loader.
 template <int DT>
 int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail &tail, int mode, hipStream_t stream) {
     constexpr int FULL = Elem<DT>::kVec;
@@ -367,7 +359,7 @@ int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail 
     if constexpr (DT != CC1D_F32) {
         if (mode == 2) return launch_width<DT, HALF, 2>(p, g, tail, stream);
     }
-    return launch_width<DT, FULL, 0>(p, g, tail, stream);
+    return launch_width<DT, HALF, 0>(p, g, tail, stream);
 }
 
 }  // namespace
@@ -395,11 +387,11 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     // Channels per lane: 2 (4 bytes of 16-bit data, 8 bytes of fp32).  A fraction of the registers
     // of a 16-byte lane, so more waves per SIMD to overlap compute with memory; measured 9 %
     // (8-byte lanes) and another 7 % (4-byte lanes) faster at the prefill shape.
-    // fwd_cl_half_vec = -1 selects 16-byte lanes.
+    // fwd_cl_half_vec = -1 forces the general tap loader.
     const int full = vec_elems(p.x_dtype);
     int mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     if (tunables().fwd_cl_half_vec < 0) mode = 0;
-    const int ch = mode == 0 ? full : p.x_dtype == CC1D_F32 ? full / 2 : CC1D_FWD_CL_CH16;
+    const int ch = p.x_dtype == CC1D_F32 ? full / 2 : CC1D_FWD_CL_CH16;
     FwdClGeom g;
     g.n_colgroups = p.dim / ch;
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;

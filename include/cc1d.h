@@ -233,7 +233,8 @@ int cc1d_abi_version(void);
 /* Benchmarking hooks: override a launch heuristic (0 restores the built-in choice).
  * Process-global, not thread-safe, meant for sweeps only.  Known names:
  *   "fwd_cl_rows"   rows of seqlen walked by one lane of the channel-last forward
- *   "fwd_cl_half_vec" -1 = lanes of the channel-last forward own 16-byte vectors (default: 2 channels)
+ *   "fwd_cl_half_vec" -1 = the channel-last forward reads its taps with the general loader even
+ *                   when they are packed
  *   "bwd_cl_rows"   same for the channel-last backward
  *   "fwd_cf_vecs"   16-byte vectors per wave segment in the channel-first forward
  *   "bwd_cf_parts"  partitions of (batch x seqlen) per channel in the channel-first backward

@@ -147,8 +147,8 @@ def test_fwd_chunking_is_bit_exact_at_prefill_size(pkg, gpu_device):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_fwd_launch_geometry_does_not_change_results(pkg, gpu_device, cc1d_lib, dtype):
-    """Every run length and both lane widths (16- and 8-byte vectors) of the channel-last
-    walk give the same bits, with seq_idx, padding, initial and final states."""
+    """Every run length and both tap loaders (packed and general) of the channel-last walk give
+    the same bits, with seq_idx, padding, initial and final states."""
     lib = cabi.declare(cc1d_lib)
     g = gen(11)
     x = make_x(2, 264, 333, dtype, True, g).to(gpu_device)
