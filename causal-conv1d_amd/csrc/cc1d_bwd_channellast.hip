@@ -52,7 +52,6 @@ struct BwdClGeom {
     uint32_t waves_per_row;   // ceil(n_colgroups / 64): workgroups side by side on one row
     uint32_t total;           // batch * n_quads * waves_per_row workgroups
     uint32_t blocks_per_xcd;  // grid size / 8
-    int32_t w_fast;           // weights_contiguous_f32
     int32_t w_mode;           // weights_mode: 0 general loader, 1 / 2 packed taps
 };
 
@@ -79,8 +78,9 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
     // halo rows and the first row groups have been requested as well.
     float wv[CH][W], bv[CH];
     PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
+    StridedTaps<W, CH> any_taps;
     if (WM != 0) taps.request(p.weight, p.bias, c0);
-    else load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, g.w_fast != 0, c0, wv, bv);
+    else any_taps.request(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, c0);
 
     // Row pointers of this run; offsets inside a run fit 32 bits (checked by the launcher).
     const char *xrun = reinterpret_cast<const char *>(reinterpret_cast<const T_ *>(p.x) + (int64_t)b * p.x_stride_b + c0 + (int64_t)t0 * p.x_stride_l);
@@ -164,6 +164,7 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
     }
     auto fill_windows = [&]() __attribute__((always_inline)) {
         if (WM != 0) taps.finish(p.bias != nullptr, wv, bv);
+        else any_taps.finish(p.w_dtype, p.bias != nullptr, wv, bv);
         float xh[2 * (W - 1)][CH];
 #pragma unroll
         for (int q = 0; q < 2 * (W - 1); ++q) P::unpack(xh_raw[q], xh[q]);
@@ -516,7 +517,6 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     if (total * kBlock >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
     g.total = (uint32_t)total;
     g.blocks_per_xcd = (uint32_t)((total + kXcds - 1) / kXcds);
-    g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
     g.w_mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     return true;
 }

@@ -338,6 +338,54 @@ struct PackedTaps {
     }
 };
 
+// The same two-phase protocol for taps of any stride and of runtime element type (fp32, fp16,
+// bf16): request() fetches each tap and bias element as raw bits (one 4- or 2-byte load each,
+// under a branch on the type that is uniform for the launch) and uses none of them; finish()
+// converts.
+template <int W, int NCH>
+struct StridedTaps {
+    uint32_t wraw[NCH * W];
+    uint32_t braw[NCH];
+
+    __device__ __forceinline__ void request(const void *weight, const void *bias, int w_dtype, int64_t stride_c,
+                                            int64_t stride_w, int c0) {
+        if (w_dtype == CC1D_F32) {
+            const uint32_t *wp = reinterpret_cast<const uint32_t *>(weight);
+            const uint32_t *bp = reinterpret_cast<const uint32_t *>(bias != nullptr ? bias : weight);
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+#pragma unroll
+                for (int w = 0; w < W; ++w) wraw[j * W + w] = wp[(int64_t)(c0 + j) * stride_c + w * stride_w];
+                braw[j] = bias != nullptr ? bp[c0 + j] : 0u;
+            }
+        } else {
+            const uint16_t *wp = reinterpret_cast<const uint16_t *>(weight);
+            const uint16_t *bp = reinterpret_cast<const uint16_t *>(bias != nullptr ? bias : weight);
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+#pragma unroll
+                for (int w = 0; w < W; ++w) wraw[j * W + w] = wp[(int64_t)(c0 + j) * stride_c + w * stride_w];
+                braw[j] = bias != nullptr ? bp[c0 + j] : 0u;
+            }
+        }
+    }
+    static __device__ __forceinline__ float as_float(uint32_t bits, int w_dtype) {
+        if (w_dtype == CC1D_F32) return bitcast<float>(bits);
+        if (w_dtype == CC1D_BF16) return bitcast<float>(bits << 16);
+        return (float)bitcast<_Float16>((uint16_t)bits);
+    }
+    __device__ __forceinline__ void finish(int w_dtype, bool has_bias, float (&wv)[NCH][W], float (&bv)[NCH]) {
+#pragma unroll
+        for (int i = 0; i < NCH * W; ++i) asm volatile("" : "+v"(wraw[i]));
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) asm volatile("" : "+v"(braw[j]));
+#pragma unroll
+        for (int i = 0; i < NCH * W; ++i) wv[i / W][i % W] = as_float(wraw[i], w_dtype);
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) bv[j] = has_bias ? as_float(braw[j], w_dtype) : 0.f;
+    }
+};
+
 // ---------------------------------------------------------------------------------
 // Wave64 lane shifts through DPP (no LDS, no memory).  All 64 lanes must be active.
 //   from_prev_lane: lane i receives lane i-1's value, lane 0 receives `lane0_fill`.

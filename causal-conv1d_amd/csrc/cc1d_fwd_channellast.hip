@@ -52,7 +52,6 @@ struct FwdClGeom {
     uint32_t waves_per_row;   // ceil(n_colgroups / 64): wavefronts side by side on one row
     uint32_t total;           // batch * n_runs * waves_per_row wavefronts
     uint32_t blocks_per_xcd;  // grid size / 8
-    int32_t w_fast;           // weights_contiguous_f32
 };
 
 // WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
@@ -98,13 +97,15 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     constexpr bool SCALED = SILU && !PRECISE;
     float wv[CH][W], bv[CH];
     PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)> taps;
+    StridedTaps<W, CH> any_taps;
     if (WFAST) taps.request(p.weight, p.bias, c0);
-    else load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, g.w_fast != 0, c0, wv, bv);
+    else any_taps.request(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, c0);
     // 16-bit outputs with SiLU: taps and bias carry the factor -log2(e), so the sums below
     // are already the exponent the activation needs (see silu_from_scaled).  Applied by
     // prepare(), after the first row groups have been requested.
     auto scale_taps = [&]() {
         if (WFAST) taps.finish(p.bias != nullptr, wv, bv);
+        else any_taps.finish(p.w_dtype, p.bias != nullptr, wv, bv);
         if (SCALED) {
 #pragma unroll
             for (int j = 0; j < CH; ++j) {
@@ -404,7 +405,6 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     g.total = (uint32_t)total;
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
-    g.w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
     VarlenTail tail = {};
     tail.first_block = g.blocks_per_xcd * kXcds;
     if (gather != nullptr) {
