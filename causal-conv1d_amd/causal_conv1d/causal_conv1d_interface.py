@@ -14,6 +14,7 @@ channel-first x (the reference asserts channel-last, :39-42).
 import torch
 
 from causal_conv1d.cpp_functions import (
+    _causal_conv1d_update_out_cpp,
     _states_like,
     causal_conv1d_bwd_function,
     causal_conv1d_fwd_function,
@@ -137,11 +138,8 @@ def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cach
     row conv_state_indices[b]; a negative index gives zeros and leaves the cache alone.
     Returns out shaped like x.
     """
-    silu = _wants_silu(activation)
-    single = x.dim() == 2
-    out = causal_conv1d_update_function(x.unsqueeze(-1) if single else x, conv_state, weight, bias,
-                                        silu, cache_seqlens, conv_state_indices)
-    return out.squeeze(-1) if single else out
+    return _causal_conv1d_update_out_cpp(x, conv_state, weight, bias, _wants_silu(activation), cache_seqlens,
+                                         conv_state_indices)
 
 
 def causal_conv1d_update_ref(x, conv_state, weight, bias=None, activation=None, cache_seqlens=None):

@@ -25,6 +25,9 @@ _causal_conv1d_update_cpp = torch.ops.DaoAILab._causal_conv1d_update_cpp
 # Not an op of the reference: the backward with dweight / dbias as plain outputs, so that the
 # wrapper below does not have to zero-fill them first (two small launches per backward call).
 _causal_conv1d_bwd_overwrite_cpp = torch.ops.DaoAILab._causal_conv1d_bwd_overwrite_cpp
+# Also not an op of the reference: the decode step for x (batch, dim) or (batch, dim, seqlen) with
+# the result allocated in C++, so that causal_conv1d_update is a single dispatcher hop.
+_causal_conv1d_update_out_cpp = torch.ops.DaoAILab._causal_conv1d_update_out_cpp
 
 
 def _states_like(x: Tensor, width: int) -> Tensor:

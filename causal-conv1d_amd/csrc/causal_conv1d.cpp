@@ -243,14 +243,20 @@ void causal_conv1d_update(const at::Tensor &x, const at::Tensor &conv_state, con
                 "tensors must be on the GPU");
     TORCH_CHECK(conv_state.scalar_type() == x.scalar_type(), "conv_state must have the dtype of x");
     TORCH_CHECK(out.scalar_type() == x.scalar_type(), "out must have the dtype of x");
-    TORCH_CHECK(x.dim() == 3, "x must be (batch, dim, seqlen)");
+    // x and out may also be (batch, dim): one token, no seqlen axis.
+    const bool flat = x.dim() == 2;
+    TORCH_CHECK(flat || x.dim() == 3, "x must be (batch, dim, seqlen)");
     TORCH_CHECK(conv_state.dim() == 3, "conv_state must be (batch, dim, state_len)");
-    const int64_t batch = x.size(0), dim = x.size(1), seqlen = x.size(2);
+    const int64_t batch = x.size(0), dim = x.size(1), seqlen = flat ? 1 : x.size(2);
     const int64_t width = weight.size(-1);
     const int64_t state_len = conv_state.size(2);
     TORCH_CHECK(state_len >= width - 1, "conv_state length must be at least width - 1");
     CHECK_SHAPE(weight, dim, width);
-    CHECK_SHAPE(out, batch, dim, seqlen);
+    if (flat) {
+        CHECK_SHAPE(out, batch, dim);
+    } else {
+        CHECK_SHAPE(out, batch, dim, seqlen);
+    }
     check_bias(bias_, weight.scalar_type(), dim);
 
     cc1d_update_params p = {};
@@ -262,7 +268,7 @@ void causal_conv1d_update(const at::Tensor &x, const at::Tensor &conv_state, con
     p.w_dtype = to_cc1d_dtype(weight.scalar_type(), "weight");
     p.silu = silu_activation ? 1 : 0;
     p.x = x.data_ptr();
-    p.x_stride_b = x.stride(0); p.x_stride_c = x.stride(1); p.x_stride_l = x.stride(2);
+    p.x_stride_b = x.stride(0); p.x_stride_c = x.stride(1); p.x_stride_l = flat ? dim : x.stride(2);
     p.conv_state = conv_state.data_ptr();
     p.state_stride_b = conv_state.stride(0); p.state_stride_c = conv_state.stride(1);
     p.state_stride_l = conv_state.stride(2);
@@ -270,7 +276,7 @@ void causal_conv1d_update(const at::Tensor &x, const at::Tensor &conv_state, con
     p.w_stride_c = weight.stride(0); p.w_stride_w = weight.stride(1);
     p.bias = bias_.has_value() ? bias_.value().data_ptr() : nullptr;
     p.out = out.data_ptr();
-    p.out_stride_b = out.stride(0); p.out_stride_c = out.stride(1); p.out_stride_l = out.stride(2);
+    p.out_stride_b = out.stride(0); p.out_stride_c = out.stride(1); p.out_stride_l = flat ? dim : out.stride(2);
 
     if (conv_state_indices_.has_value()) {
         const auto &idx = conv_state_indices_.value();
@@ -391,6 +397,24 @@ void update_op(const at::Tensor &x, at::Tensor &conv_state, const at::Tensor &we
     causal_conv1d_update(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices);
 }
 
+// The decode step as the user-facing function needs it: x (batch, dim) or (batch, dim, seqlen),
+// the result allocated here and shaped like x.  One dispatcher hop instead of the wrapper's
+// unsqueeze / empty_like / op / squeeze in Python, which cost more host time than the kernel
+// runs.  Not an op of the reference.
+at::Tensor update_out_op(const at::Tensor &x, at::Tensor &conv_state, const at::Tensor &weight,
+                         const std::optional<at::Tensor> &bias, bool silu_activation,
+                         const std::optional<at::Tensor> &cache_seqlens,
+                         const std::optional<at::Tensor> &conv_state_indices) {
+    TORCH_CHECK(x.dim() == 2 || x.dim() == 3, "x must be (batch, dim) or (batch, dim, seqlen)");
+    at::Tensor out = at::empty_like(x);
+    causal_conv1d_update(x, conv_state, weight, bias, out, silu_activation, cache_seqlens, conv_state_indices);
+    return out;
+}
+at::Tensor update_out_meta(const at::Tensor &x, at::Tensor &, const at::Tensor &, const std::optional<at::Tensor> &,
+                           bool, const std::optional<at::Tensor> &, const std::optional<at::Tensor> &) {
+    return at::empty_like(x);
+}
+
 // Shape propagation has nothing to do: every output is an argument.
 void fwd_meta(const at::Tensor &, const at::Tensor &, const std::optional<at::Tensor> &,
               const std::optional<at::Tensor> &, const std::optional<at::Tensor> &, at::Tensor &,
@@ -425,6 +449,9 @@ TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {
           "Tensor? initial_states, Tensor(a!)? dfinal_states, Tensor(b!) dx, Tensor(c!) dweight, "
           "Tensor(d!)? dbias, Tensor(e!)? dinitial_states, bool silu_activation) -> ()",
           {at::Tag::pt2_compliant_tag});
+    m.def("_causal_conv1d_update_out_cpp(Tensor x, Tensor(a!) conv_state, Tensor weight, Tensor? bias, "
+          "bool silu_activation, Tensor? cache_seqlens, Tensor? conv_state_indices) -> Tensor",
+          {at::Tag::pt2_compliant_tag});
     m.def("_causal_conv1d_update_cpp(Tensor x, Tensor(a!) conv_state, Tensor weight, Tensor? bias, "
           "Tensor(b!) out, bool silu_activation, Tensor? cache_seqlens, Tensor? conv_state_indices) -> ()",
           {at::Tag::pt2_compliant_tag});
@@ -436,6 +463,7 @@ TORCH_LIBRARY_IMPL(DaoAILab, CompositeExplicitAutograd, m) {
     m.impl("_causal_conv1d_bwd_cpp", &bwd_op);
     m.impl("_causal_conv1d_bwd_overwrite_cpp", &bwd_overwrite_op);
     m.impl("_causal_conv1d_update_cpp", &update_op);
+    m.impl("_causal_conv1d_update_out_cpp", &update_out_op);
 }
 
 TORCH_LIBRARY_IMPL(DaoAILab, Meta, m) {
@@ -443,4 +471,5 @@ TORCH_LIBRARY_IMPL(DaoAILab, Meta, m) {
     m.impl("_causal_conv1d_bwd_cpp", &bwd_meta);
     m.impl("_causal_conv1d_bwd_overwrite_cpp", &bwd_meta);
     m.impl("_causal_conv1d_update_cpp", &update_meta);
+    m.impl("_causal_conv1d_update_out_cpp", &update_out_meta);
 }

@@ -64,6 +64,10 @@ def test_opcheck_update(pkg, gpu_device):
     idx = torch.tensor([3, 0, -1, 5], dtype=torch.int32, device=dev)
     op = torch.ops.DaoAILab._causal_conv1d_update_cpp
     torch.library.opcheck(op, (x, state, w.to(dev), b.to(dev), out, True, cache, idx), test_utils=OPCHECKS)
+    # the variant causal_conv1d_update uses: result allocated by the op, x (batch, dim) allowed
+    op = torch.ops.DaoAILab._causal_conv1d_update_out_cpp
+    torch.library.opcheck(op, (x, state, w.to(dev), b.to(dev), True, cache, idx), test_utils=OPCHECKS)
+    torch.library.opcheck(op, (x[:, :, 0], state, w.to(dev), b.to(dev), False, None, idx), test_utils=OPCHECKS)
 
 
 def test_compile_fn_forward_backward_matches_eager(pkg, gpu_device):
