@@ -35,6 +35,26 @@ def _kernel_layout(t):
     return t if 1 in (t.stride(1), t.stride(2)) else t.contiguous()
 
 
+def _forward(x, weight, bias, seq_idx, initial_states, return_final_states, final_states_out, silu):
+    """Checks, layouts and the device call of the forward; returns what backward needs too."""
+    x = _kernel_layout(x)
+    bias = None if bias is None else bias.contiguous()
+    if seq_idx is not None:
+        assert initial_states is None, "initial_states must be None if seq_idx is not None"
+        assert not return_final_states, "If seq_idx is not None, we don't return final_states_out"
+        seq_idx = seq_idx.contiguous()
+    if initial_states is not None:
+        initial_states = _kernel_layout(initial_states)
+    if not return_final_states:
+        final_states_out = None
+    elif final_states_out is None:
+        final_states_out = _states_like(x, weight.shape[1])
+    else:
+        assert 1 in (final_states_out.stride(1), final_states_out.stride(2))
+    out = causal_conv1d_fwd_function(x, weight, bias, seq_idx, initial_states, final_states_out, silu)
+    return out, final_states_out, (x, weight, bias, seq_idx, initial_states)
+
+
 class CausalConv1dFn(torch.autograd.Function):
     """Forward and backward through the device ops; saves only the inputs (the pre-activation
     is recomputed in backward)."""
@@ -43,25 +63,12 @@ class CausalConv1dFn(torch.autograd.Function):
     def forward(ctx, x, weight, bias=None, seq_idx=None, initial_states=None,
                 return_final_states=False, final_states_out=None, activation=None):
         silu = _wants_silu(activation)
-        x = _kernel_layout(x)
-        bias = None if bias is None else bias.contiguous()
-        if seq_idx is not None:
-            assert initial_states is None, "initial_states must be None if seq_idx is not None"
-            assert not return_final_states, "If seq_idx is not None, we don't return final_states_out"
-            seq_idx = seq_idx.contiguous()
-        if initial_states is not None:
-            initial_states = _kernel_layout(initial_states)
-        if not return_final_states:
-            final_states_out = None
-        elif final_states_out is None:
-            final_states_out = _states_like(x, weight.shape[1])
-        else:
-            assert 1 in (final_states_out.stride(1), final_states_out.stride(2))
-        out = causal_conv1d_fwd_function(x, weight, bias, seq_idx, initial_states, final_states_out, silu)
-        ctx.save_for_backward(x, weight, bias, seq_idx, initial_states)
+        out, final_states_out, saved = _forward(x, weight, bias, seq_idx, initial_states, return_final_states,
+                                                final_states_out, silu)
+        ctx.save_for_backward(*saved)
         ctx.activation = silu
         ctx.return_final_states = return_final_states
-        ctx.return_dinitial_states = initial_states is not None and initial_states.requires_grad
+        ctx.return_dinitial_states = saved[4] is not None and saved[4].requires_grad
         return (out, final_states_out) if return_final_states else out
 
     @staticmethod
@@ -88,6 +95,15 @@ def causal_conv1d_fn(x, weight, bias=None, seq_idx=None, initial_states=None,
     (out, final_states), final_states (batch, dim, width-1) written to final_states_out if given.
     activation: None, "silu" or "swish".
     """
+    wants_grad = torch.is_grad_enabled() and (
+        x.requires_grad or weight.requires_grad or (bias is not None and bias.requires_grad)
+        or (initial_states is not None and initial_states.requires_grad))
+    if not wants_grad:
+        # Inference: no graph to record, so no autograd.Function around the call (it costs 3.5 us
+        # of host time, as much as the kernel at small shapes).
+        out, final_states_out, _ = _forward(x, weight, bias, seq_idx, initial_states, return_final_states,
+                                            final_states_out, _wants_silu(activation))
+        return (out, final_states_out) if return_final_states else out
     return CausalConv1dFn.apply(x, weight, bias, seq_idx, initial_states, return_final_states,
                                 final_states_out, activation)
 
