@@ -1,7 +1,7 @@
 // Decode-step update for gfx950.  Takes over causal_conv1d_update_kernel and its
 // launcher (csrc/causal_conv1d_update.cu:23-136 of the reference).
 //
-// Three kernels:
+// Four kernels:
 //  * update_step_kernel — the decode step proper: one new token (seqlen 1) and x, out,
 //    conv_state with unit stride along dim.  A lane owns one 8-byte vector of channels of
 //    two consecutive batch entries; all of its loads (window rows, x) are issued before
@@ -10,6 +10,9 @@
 //    This shape moves about 22 MB; its
 //    run time is within a microsecond of a plain copy of the same footprint, which itself
 //    only costs about 1.6 us more than an empty launch.
+//  * update_tokens_kernel — 2 to 8 new tokens a call (speculative decoding), same layout and
+//    lane width: one batch entry per lane, every x row and the window requested up front,
+//    taps through LDS, the tokens then produced in order from registers.
 //  * update_vec_kernel — any seqlen, same unit-stride layout (the
 //    layout Mamba-style decoders allocate: (batch, state_len, dim) in memory).  A lane
 //    owns one 16-byte vector of channels; every state row, x row and out row moves as
