@@ -158,10 +158,21 @@ struct StepArgs {
 // owns kTapUnits consecutive 8-byte units in memory; request() has every thread fetch one
 // 16-byte pair of units per trip (one unit when a column group has an odd number of them) and
 // one unit of the bias, publish() parks them as staged[unit][lane] (read back without bank
-// conflicts), and after a barrier collect() gives a lane its own.  Callers issue request()
+// conflicts; see CC1D_TAPS_PAD for the writes), and after a barrier collect() gives a lane its own.  Callers issue request()
 // first and their data loads right behind it, so the LDS round trip happens while the data is
 // in flight.
 constexpr int kStepWaves = kBlock / kWave;
+// Extra 8-byte entries per row of the staging array.  collect() reads a row lane by lane and
+// never conflicts; publish() writes a thread's units into rows 1 KiB apart, a 4-way bank
+// conflict: SQ_LDS_BANK_CONFLICT counts 69,888 cycles per decode launch over the whole chip
+// (273 per CU) out of 204,288 LDS-active cycles.  A pad of 2 entries spreads the rows over the
+// 32 banks (5,376 conflict cycles left, from the bias rows) but the row stride is then no power
+// of two, and the launch measured 0.05 us slower (4.66 against 4.61 us) five times out of five:
+// the conflicts are not on the critical path, the address arithmetic is.  Hence 0.
+#ifndef CC1D_TAPS_PAD
+#define CC1D_TAPS_PAD 0
+#endif
+constexpr int kTapRow = kWave + CC1D_TAPS_PAD;
 
 template <class Taps, int CH, int W>
 struct WorkgroupTaps {
@@ -198,7 +209,7 @@ struct WorkgroupTaps {
         if (bias != nullptr && threadIdx.x < cols_here * (uint32_t)kBiasUnits)
             bias_unit = reinterpret_cast<const u32x2 *>(bsrc)[threadIdx.x];
     }
-    __device__ __forceinline__ void publish(u32x2 (&staged)[kUnits][kWave]) const {
+    __device__ __forceinline__ void publish(u32x2 (&staged)[kUnits][kTapRow]) const {
 #pragma unroll
         for (int q = 0; q < kTrips; ++q) {
             const uint32_t pi = (uint32_t)q * kBlock + threadIdx.x;
@@ -212,7 +223,7 @@ struct WorkgroupTaps {
         if (threadIdx.x < (uint32_t)(kWave * kBiasUnits))
             staged[kTapUnits + threadIdx.x % kBiasUnits][threadIdx.x / kBiasUnits] = bias_unit;
     }
-    static __device__ __forceinline__ void collect(const u32x2 (&staged)[kUnits][kWave], uint32_t lane, Taps &taps) {
+    static __device__ __forceinline__ void collect(const u32x2 (&staged)[kUnits][kTapRow], uint32_t lane, Taps &taps) {
 #pragma unroll
         for (int u = 0; u < kTapUnits; ++u) {
             const u32x2 v = staged[u][lane];
@@ -241,7 +252,7 @@ update_step_kernel(const StepArgs a) {
     using Taps = PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)>;
     constexpr bool PRECISE = E::kPreciseAct;
     using Staging = WorkgroupTaps<Taps, CH, W>;
-    __shared__ u32x2 staged[Staging::kUnits][kWave];
+    __shared__ u32x2 staged[Staging::kUnits][kTapRow];
 
     const uint32_t lc = threadIdx.x & (kWave - 1);
     const int wave_row = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
@@ -355,7 +366,7 @@ update_tokens_kernel(const TokensArgs ta) {
     constexpr bool PRECISE = E::kPreciseAct;
     using Taps = PackedTaps<W, CH, (WM == 1 ? CC1D_F32 : DT)>;
     using Staging = WorkgroupTaps<Taps, CH, W>;
-    __shared__ u32x2 staged[Staging::kUnits][kWave];
+    __shared__ u32x2 staged[Staging::kUnits][kTapRow];
     const StepArgs &a = ta.s;
 
     const uint32_t lc = threadIdx.x & (kWave - 1);
