@@ -369,10 +369,19 @@ int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail 
 // runs put more wavefronts in flight, which is what keeps HBM busy while other waves
 // compute, and spread the work more evenly over the CUs.  32 rows measured best at the
 // prefill shape (8 x 2048 rows x 5376 channels); short sequences take what they have.
-static int choose_rows_per_run(int seqlen, int64_t row_bytes) {
+// A launch that fills the chip's wavefront slots (256 CUs x 4 SIMDs x `waves_per_simd`) less than
+// 0.6 times over with 32-row runs is bound by the length of a wavefront's own chain of loads,
+// not by bandwidth, and takes 16-row runs: 3.7 against 4.6 us at (1, 5376, 64) bf16, 5.5 against
+// 6.2 us at (1, 5376, 1024), 8.6 against 9.5 us at (1, 5376, 1024) fp32; from about one fill
+// upwards 32 rows are as good or better.
+static int choose_rows_per_run(int seqlen, int64_t row_bytes, int64_t waves_per_row_of_runs, int waves_per_simd) {
     constexpr int U = 2 * CC1D_FWD_CL_UNROLL;         // the walk is unrolled over two groups
     int T = tunables().fwd_cl_rows;
-    if (T <= 0) T = 32;
+    if (T <= 0) {
+        T = 32;
+        const int64_t waves32 = waves_per_row_of_runs * ((seqlen + 31) / 32);
+        if (10 * waves32 <= 6 * (int64_t)(256 * 4) * waves_per_simd) T = 16;
+    }
     const int cap = (seqlen + U - 1) / U * U;          // never longer than the sequence
     if (T > cap) T = cap;
     T = (T + U - 1) / U * U;
@@ -396,10 +405,11 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     FwdClGeom g;
     g.n_colgroups = p.dim / ch;
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
-    g.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * elem_bytes(p.x_dtype));
+    g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
+    g.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * elem_bytes(p.x_dtype), (int64_t)p.batch * g.waves_per_row,
+                                         p.x_dtype == CC1D_F32 ? CC1D_FWD_CL_OCC8 : CC1D_FWD_CL_OCC4);
     if (g.rows_per_run == 0) return CC1D_ERR_TOO_LARGE;
     g.n_runs = (p.seqlen + g.rows_per_run - 1) / g.rows_per_run;
-    g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
     const int64_t total = (int64_t)p.batch * g.n_runs * g.waves_per_row;
     if (total * kWave >= ((int64_t)1 << 31) - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
     g.total = (uint32_t)total;
