@@ -25,6 +25,9 @@ _causal_conv1d_update_cpp = torch.ops.DaoAILab._causal_conv1d_update_cpp
 # Not an op of the reference: the backward with dweight / dbias as plain outputs, so that the
 # wrapper below does not have to zero-fill them first (two small launches per backward call).
 _causal_conv1d_bwd_overwrite_cpp = torch.ops.DaoAILab._causal_conv1d_bwd_overwrite_cpp
+# Not an op of the reference either: the forward with `out` allocated in C++ (in x's layout) and
+# returned, which saves the wrapper's empty_like.
+_causal_conv1d_fwd_out_cpp = torch.ops.DaoAILab._causal_conv1d_fwd_out_cpp
 # Also not an op of the reference: the decode step for x (batch, dim) or (batch, dim, seqlen) with
 # the result allocated in C++, so that causal_conv1d_update is a single dispatcher hop.
 _causal_conv1d_update_out_cpp = torch.ops.DaoAILab._causal_conv1d_update_out_cpp
@@ -42,10 +45,8 @@ def _states_like(x: Tensor, width: int) -> Tensor:
 
 def causal_conv1d_fwd_function(x: Tensor, weight: Tensor, bias: _Opt, seq_idx: _Opt, initial_states: _Opt,
                                final_states_out: _Opt, silu_activation: bool) -> Tensor:
-    """Allocates `out` in x's layout and fills it; `final_states_out`, if given, is filled too."""
-    out = torch.empty_like(x)
-    _causal_conv1d_fwd_cpp(x, weight, bias, seq_idx, initial_states, out, final_states_out, silu_activation)
-    return out
+    """Returns `out`, allocated in x's layout; `final_states_out`, if given, is filled too."""
+    return _causal_conv1d_fwd_out_cpp(x, weight, bias, seq_idx, initial_states, final_states_out, silu_activation)
 
 
 def causal_conv1d_bwd_function(x: Tensor, weight: Tensor, bias: _Opt, dout: Tensor, seq_idx: _Opt,

@@ -366,6 +366,23 @@ void fwd_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<a
     causal_conv1d_fwd(x, weight, bias, seq_idx, initial_states, out, fin, silu_activation);
 }
 
+// The forward with its result allocated here, in x's layout: one dispatcher hop and no
+// empty_like in Python (about a microsecond of host time, which is what a short prefill is
+// bound by).  Not an op of the reference.
+at::Tensor fwd_out_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<at::Tensor> &bias,
+                      const std::optional<at::Tensor> &seq_idx, const std::optional<at::Tensor> &initial_states,
+                      const std::optional<at::Tensor> &final_states_out, bool silu_activation) {
+    at::Tensor out = at::empty_like(x);
+    std::optional<at::Tensor> fin = final_states_out;
+    causal_conv1d_fwd(x, weight, bias, seq_idx, initial_states, out, fin, silu_activation);
+    return out;
+}
+at::Tensor fwd_out_meta(const at::Tensor &x, const at::Tensor &, const std::optional<at::Tensor> &,
+                        const std::optional<at::Tensor> &, const std::optional<at::Tensor> &,
+                        const std::optional<at::Tensor> &, bool) {
+    return at::empty_like(x);
+}
+
 void bwd_op(const at::Tensor &x, const at::Tensor &weight, const std::optional<at::Tensor> &bias,
             const at::Tensor &dout, const std::optional<at::Tensor> &seq_idx,
             const std::optional<at::Tensor> &initial_states, const std::optional<at::Tensor> &dfinal_states,
@@ -441,6 +458,9 @@ TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {
     m.def("_causal_conv1d_fwd_cpp(Tensor x, Tensor weight, Tensor? bias, Tensor? seq_idx, "
           "Tensor? initial_states, Tensor(a!) out, Tensor(b!)? final_states_out, bool silu_activation) -> ()",
           {at::Tag::pt2_compliant_tag});
+    m.def("_causal_conv1d_fwd_out_cpp(Tensor x, Tensor weight, Tensor? bias, Tensor? seq_idx, "
+          "Tensor? initial_states, Tensor(a!)? final_states_out, bool silu_activation) -> Tensor",
+          {at::Tag::pt2_compliant_tag});
     m.def("_causal_conv1d_bwd_cpp(Tensor x, Tensor weight, Tensor? bias, Tensor dout, Tensor? seq_idx, "
           "Tensor? initial_states, Tensor(a!)? dfinal_states, Tensor(b!) dx, Tensor(c!) dweight, "
           "Tensor(d!)? dbias, Tensor(e!)? dinitial_states, bool silu_activation) -> ()",
@@ -460,6 +480,7 @@ TORCH_LIBRARY_FRAGMENT(DaoAILab, m) {
 // One kernel for every real backend: on anything but the GPU it raises (there is no host path).
 TORCH_LIBRARY_IMPL(DaoAILab, CompositeExplicitAutograd, m) {
     m.impl("_causal_conv1d_fwd_cpp", &fwd_op);
+    m.impl("_causal_conv1d_fwd_out_cpp", &fwd_out_op);
     m.impl("_causal_conv1d_bwd_cpp", &bwd_op);
     m.impl("_causal_conv1d_bwd_overwrite_cpp", &bwd_overwrite_op);
     m.impl("_causal_conv1d_update_cpp", &update_op);
@@ -468,6 +489,7 @@ TORCH_LIBRARY_IMPL(DaoAILab, CompositeExplicitAutograd, m) {
 
 TORCH_LIBRARY_IMPL(DaoAILab, Meta, m) {
     m.impl("_causal_conv1d_fwd_cpp", &fwd_meta);
+    m.impl("_causal_conv1d_fwd_out_cpp", &fwd_out_meta);
     m.impl("_causal_conv1d_bwd_cpp", &bwd_meta);
     m.impl("_causal_conv1d_bwd_overwrite_cpp", &bwd_meta);
     m.impl("_causal_conv1d_update_cpp", &update_meta);

@@ -34,6 +34,10 @@ def test_opcheck_fwd(pkg, gpu_device):
     seq = torch.zeros(2, 96, dtype=torch.int32, device=gpu_device)
     seq[:, 40:] = 1
     torch.library.opcheck(op, (x, w, None, seq, None, out, None, False), test_utils=OPCHECKS)
+    # the variant the Python layer uses: out allocated by the op and returned
+    op = torch.ops.DaoAILab._causal_conv1d_fwd_out_cpp
+    torch.library.opcheck(op, (x, w, b, None, init, fin, True), test_utils=OPCHECKS)
+    torch.library.opcheck(op, (x, w, None, seq, None, None, False), test_utils=OPCHECKS)
 
 
 def test_opcheck_bwd(pkg, gpu_device):
