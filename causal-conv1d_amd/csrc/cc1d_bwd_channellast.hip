@@ -499,7 +499,16 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     // before), a workgroup's partial sums are one plane per 128 rows, and the prefill shape
     // launches 10752 wavefronts.  Measured there against 16, 24, 48, 64 and 128 rows, with and
     // without seq_idx.
-    if (T <= 0) T = 32;
+    // A launch that fills the chip's wavefront slots less than 0.1 times over with 32-row runs is
+    // bound by the length of one wavefront's chain and takes 8-row runs: (1, 5376, 64) bf16 8.1
+    // against 10.0 us, (1, 2560, 256) fp32 8.2 against 10.5 us, second stage included; from 0.16
+    // fills upwards 32 rows are as good or better.
+    if (T <= 0) {
+        T = 32;
+        const int64_t waves32 = (int64_t)p.batch * ((p.seqlen + 31) / 32) * ((g.n_colgroups + kWave - 1) / kWave);
+        const int64_t slots = (int64_t)256 * 4 * (p.x_dtype == CC1D_F32 ? 2 : CC1D_BWD_CL_OCC);
+        if (10 * waves32 <= slots) T = 8;
+    }
     const int cap = (p.seqlen + U2 - 1) / U2 * U2;     // never longer than the sequence
     if (T > cap) T = cap;
     T = (T + U2 - 1) / U2 * U2;
