@@ -64,6 +64,31 @@ def test_fwd_matches_oracle(pkg, gpu_device, dim, seqlen, dtype, channel_last, w
     assert_close(got, ref, dtype, "out")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seqlen", [4, 8, 24, 40, 72, 136, 248, 256, 264, 512])
+def test_fwd_channel_first_short_rows(pkg, gpu_device, seqlen, dtype):
+    """Channel-first rows of at most 64 whole 16-byte vectors share a wavefront (8, 4, 2 or 1 rows
+    each): a row count that does not fill the last wavefront, every vector count class, states
+    in and out, and against the same rows one element longer (which take the walking kernel)."""
+    dev = gpu_device
+    batch, dim, width = 3, 24, 2 + seqlen % 3
+    g = gen(1000 + seqlen)
+    x = torch.randn(batch, dim, seqlen + 1, generator=g).to(dtype)
+    w, b = make_wb(dim, width, True, g)
+    init = make_states(batch, dim, width - 1, dtype, g)
+    xs = x[:, :, :seqlen].contiguous()
+    ref, ref_fin = orc.fwd(xs, w, b, initial_states=init, return_final_states=True, activation="silu")
+    got, got_fin = pkg.causal_conv1d_fn(xs.to(dev), w.to(dev), b.to(dev), initial_states=init.to(dev),
+                                        return_final_states=True, activation="silu")
+    assert_close(got, ref, dtype, "out")
+    assert torch.equal(got_fin.cpu(), ref_fin)
+    # causality: the first seqlen outputs of the longer rows are the same numbers, bit for bit
+    longer = pkg.causal_conv1d_fn(x.to(dev), w.to(dev), b.to(dev), initial_states=init.to(dev), activation="silu")
+    assert torch.equal(longer[:, :, :seqlen], got)
+    plain = pkg.causal_conv1d_fn(xs.to(dev), w.to(dev), None)
+    assert_close(plain, orc.fwd(xs, w, None), dtype, "no bias, no activation, no states")
+
+
 @pytest.mark.parametrize("pad", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("dim,seqlen,width,has_bias,silu", [
