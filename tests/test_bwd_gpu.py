@@ -84,6 +84,38 @@ def test_bwd_matches_oracle(pkg, gpu_device, dim, seqlen, dtype, channel_last, w
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seqlen", [8, 24, 40, 72, 136, 248, 256, 264, 512])
+def test_bwd_channel_first_short_rows(pkg, gpu_device, seqlen, dtype):
+    """Channel-first rows of at most 64 whole 16-byte vectors: several batch entries share a
+    wavefront.  A batch that does not fill the last group, every vector-count class, all state
+    gradients; dx and dinitial_states must also equal, bit for bit, what the same data gives
+    when it sits one element off the 16-byte grid (which takes the walking kernel)."""
+    dev = gpu_device
+    batch, dim, width = 5, 24, 2 + seqlen % 3
+    g = gen(2000 + seqlen)
+    x = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+    dout = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+    w, b = make_wb(dim, width, True, g)
+    init = make_states(batch, dim, width - 1, dtype, g)
+    dfin = make_states(batch, dim, width - 1, dtype, g)
+    ref = orc.bwd(x, w, b, dout, initial_states=init, dfinal_states=dfin, activation="silu")
+    got = run_gpu(pkg, dev, x, w, b, dout, init=init, dfin=dfin, act="silu")
+    check(got, ref, dtype)
+
+    def off_grid(t):                                   # same values, rows one element off the grid
+        wide = torch.zeros(batch, dim, seqlen + 8, dtype=dtype)
+        wide[:, :, 1:1 + seqlen] = t
+        return wide[:, :, 1:1 + seqlen]
+    other = run_gpu(pkg, dev, off_grid(x), w, b, off_grid(dout), init=init, dfin=dfin, act="silu")
+    assert torch.equal(other[0], got[0]), "dx"
+    assert torch.equal(other[3], got[3]), "dinitial_states"
+    check(other, ref, dtype)
+    # no states, no bias, no activation
+    got = run_gpu(pkg, dev, x, w, None, dout)
+    check(got, orc.bwd(x, w, None, dout), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("dim,seqlen,width,has_bias,silu", [
     (64, 8, 2, True, True), (64, 16, 3, False, True), (64, 151, 4, True, False), (64, 372, 4, True, True),
     (64, 1134, 3, True, True), (4128, 32, 4, True, True), (4128, 128, 2, False, False),
