@@ -352,12 +352,15 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
     }
 }
 
-// Rows of at most 64 whole vectors on the 16-byte grid.  One wavefront per row would leave most
-// of its lanes idle, so a wavefront takes 64 / G rows at once, G = 8, 16, 32 or 64 lanes each: lane
-// (row, v) owns vector v of its row, takes its left halo from the previous lane through the same
+// Rows of at most 64 vectors.  One wavefront per row would leave most of its lanes idle, so a
+// wavefront takes 64 / G rows at once, G = 1, 2, 4 ... 64 lanes each (ALIGNED: whole vectors on the
+// 16-byte grid): lane (row, v) owns vector v of its row, takes its left halo from the previous lane through the same
 // DPP shift as the walk (vector 0 takes zeros or initial_states instead), and the whole launch is
 // one load and one store per lane.  Same arithmetic, in the same order, as the other kernels.
-template <int DT, int W, bool SILU>
+// ALIGNED = false: rows of any length up to 64 vectors, anywhere in memory (a contiguous tensor
+// whose seqlen is no multiple of the vector length, down to seqlen 1): the same lanes, with a
+// lane's up to VEC positions read and written element by element.
+template <int DT, int W, bool SILU, bool ALIGNED>
 __global__ void __launch_bounds__(kBlock)
 fwd_channelfirst_short_kernel(const cc1d_fwd_params p, const int n_vecs, const int lanes_log2, const uint32_t n_rows) {
     using E = Elem<DT>;
@@ -378,8 +381,21 @@ fwd_channelfirst_short_kernel(const cc1d_fwd_params p, const int n_vecs, const i
     const int64_t xrow = (int64_t)b * p.x_stride_b + (int64_t)c * p.x_stride_c;
     const int64_t orow = (int64_t)b * p.out_stride_b + (int64_t)c * p.out_stride_c;
 
+    const int L = p.seqlen;
     u32x4 raw = u32x4{0u, 0u, 0u, 0u};
-    if (mine) raw = ld_vec_nt<DT>(p.x, xrow + (int64_t)v * VEC);
+    if (ALIGNED) {
+        if (mine) raw = ld_vec_nt<DT>(p.x, xrow + (int64_t)v * VEC);
+    } else {
+        T elems[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) elems[e] = T(0.f);
+        if (mine) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                if (v * VEC + e < L) elems[e] = ld_raw<DT>(p.x, xrow + v * VEC + e);
+        }
+        __builtin_memcpy(&raw, elems, sizeof raw);
+    }
     float wv[W], bias_v;
 #pragma unroll
     for (int w = 0; w < W; ++w)
@@ -416,14 +432,27 @@ fwd_channelfirst_short_kernel(const cc1d_fwd_params p, const int n_vecs, const i
         for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
         acc[e] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
     }
-    if (mine) st_vec_nt<DT>(p.out, orow + (int64_t)v * VEC, E::pack(acc));
+    if (ALIGNED) {
+        if (mine) st_vec_nt<DT>(p.out, orow + (int64_t)v * VEC, E::pack(acc));
+    } else if (mine) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            if (v * VEC + e < L) st_elem<DT>(p.out, orow + v * VEC + e, acc[e]);
+    }
 
-    // final_states[b, c, i] = x[L-(W-1)+i] (a row of whole vectors is never shorter than W-1),
-    // bit-exact copies, by the lane that owns the row's last vector.
+    // final_states[b, c, i] = xpad[L-(W-1)+i], bit-exact copies (from initial_states or zero where
+    // the row is shorter than W-1), by the lane that owns the row's last vector.
     if (p.final_states != nullptr && mine && v == n_vecs - 1) {
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) {
-            const T e = ld_raw<DT>(p.x, xrow + (int64_t)(p.seqlen - (W - 1) + i));
+            const int t = L - (W - 1) + i;
+            T e = T(0.f);
+            if (t >= 0) {
+                e = ld_raw<DT>(p.x, xrow + t);
+            } else if (p.initial_states != nullptr) {
+                e = ld_raw<DT>(p.initial_states, (int64_t)b * p.init_stride_b + (int64_t)c * p.init_stride_c +
+                                                     (int64_t)(t + W - 1) * p.init_stride_l);
+            }
             st_raw<DT>(p.final_states, (int64_t)b * p.final_stride_b + (int64_t)c * p.final_stride_c +
                                            (int64_t)i * p.final_stride_l, e);
         }
@@ -431,24 +460,28 @@ fwd_channelfirst_short_kernel(const cc1d_fwd_params p, const int n_vecs, const i
 }
 
 template <int DT>
-int launch_short(const cc1d_fwd_params &p, int n_vecs, hipStream_t stream) {
-    const int lanes_log2 = n_vecs <= 8 ? 3 : n_vecs <= 16 ? 4 : n_vecs <= 32 ? 5 : 6;
+int launch_short(const cc1d_fwd_params &p, int n_vecs, bool aligned, hipStream_t stream) {
+    int lanes_log2 = 0;
+    while ((1 << lanes_log2) < n_vecs) ++lanes_log2;
     const int64_t rows = (int64_t)p.batch * p.dim;
     const int64_t threads = rows << lanes_log2;
     if (threads >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
     const dim3 grid((uint32_t)((threads + kBlock - 1) / kBlock)), block(kBlock);
     const uint32_t n_rows = (uint32_t)rows;
+#define CC1D_SHORT2(WIDTH, SILU_ON)                                                                                  \
+    if (aligned) hipLaunchKernelGGL((fwd_channelfirst_short_kernel<DT, WIDTH, SILU_ON, true>), grid, block, 0,       \
+                                    stream, p, n_vecs, lanes_log2, n_rows);                                           \
+    else hipLaunchKernelGGL((fwd_channelfirst_short_kernel<DT, WIDTH, SILU_ON, false>), grid, block, 0, stream, p,   \
+                            n_vecs, lanes_log2, n_rows)
 #define CC1D_SHORT(WIDTH)                                                                                             \
-    if (p.silu) hipLaunchKernelGGL((fwd_channelfirst_short_kernel<DT, WIDTH, true>), grid, block, 0, stream, p,      \
-                                   n_vecs, lanes_log2, n_rows);                                                       \
-    else hipLaunchKernelGGL((fwd_channelfirst_short_kernel<DT, WIDTH, false>), grid, block, 0, stream, p, n_vecs,    \
-                            lanes_log2, n_rows)
+    if (p.silu) { CC1D_SHORT2(WIDTH, true); } else { CC1D_SHORT2(WIDTH, false); }
     switch (p.width) {
         case 2: CC1D_SHORT(2); break;
         case 3: CC1D_SHORT(3); break;
         default: CC1D_SHORT(4); break;
     }
 #undef CC1D_SHORT
+#undef CC1D_SHORT2
     return launch_status();
 }
 
@@ -494,11 +527,15 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     const int64_t rows = (int64_t)p.batch * p.dim;
     // Short rows of whole vectors, up to eight to a wavefront, no walk: (4, 5376, 256) bf16 11.2 -> 6.0 us,
     // (8, 1024, 512) bf16 6.7 -> 4.8 us, (4, 5376, 256) fp32 10.9 -> 8.5 us, (1, 5376, 64) bf16 4.8 -> 3.3 us.
-    if (same_grid && on_grid && p.seqlen % vec == 0 && max_vecs <= 64 && tunables().fwd_cf_vecs <= 0) {
+    // Rows that are not whole vectors on one grid take the same lanes with element accesses:
+    // (16, 5376, 100) bf16 45.9 -> 25.4 us, (64, 2048, 60) 63.7 -> 16.4 us, (256, 5376, 4) 360 -> 11.9 us.
+    const int64_t short_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
+    if (short_vecs <= 64 && tunables().fwd_cf_vecs <= 0) {
+        const bool aligned = same_grid && on_grid && p.seqlen % vec == 0;
         switch (p.x_dtype) {
-            case CC1D_F32: return launch_short<CC1D_F32>(p, (int)max_vecs, stream);
-            case CC1D_F16: return launch_short<CC1D_F16>(p, (int)max_vecs, stream);
-            default: return launch_short<CC1D_BF16>(p, (int)max_vecs, stream);
+            case CC1D_F32: return launch_short<CC1D_F32>(p, (int)short_vecs, aligned, stream);
+            case CC1D_F16: return launch_short<CC1D_F16>(p, (int)short_vecs, aligned, stream);
+            default: return launch_short<CC1D_BF16>(p, (int)short_vecs, aligned, stream);
         }
     }
     int64_t vps;
