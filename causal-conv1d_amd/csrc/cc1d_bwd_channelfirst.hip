@@ -27,8 +27,9 @@
 // partly filled last step of a row are done first, one checked step at a time, and the few
 // positions of a row in front of its first whole vector or behind its last one are done one
 // per lane, straight from memory.  The general kernel takes tensors on different grids and
-// rows shorter than two vectors.  The short-row kernel takes rows of at most 64 whole vectors,
-// several batch entries of a channel to a wavefront and no walk.
+// rows longer than 64 vectors.  The short-row kernel takes rows of at most 64 vectors (whole
+// vectors on one grid, or element by element), several batch entries of a channel to a
+// wavefront and no walk.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -44,13 +45,14 @@ __device__ __forceinline__ void accumulate(float *dst, float v, int overwrite) {
 
 struct BwdCfGeom {
     int32_t streaming;        // 0: general kernel; streaming kernel with rows 1: on the 16-byte grid, 2: anywhere on it;
-                              // 3: short-row kernel (an item is then a group of batch entries, n_segs 1)
+                              // 3: short-row kernel (an item is then a group of batch entries, n_segs 1),
+                              // 4: the same with element accesses
     int32_t vecs_per_seg;     // multiple of 64
     int32_t n_segs;           // segments per row
     int32_t n_items;          // batch * n_segs
     int32_t n_parts;          // slices of the item list per channel
     int32_t items_per_part;
-    int32_t lanes_log2;       // short-row kernel (streaming == 3): log2 of the lanes one row takes
+    int32_t lanes_log2;       // short-row kernel (streaming 3, 4): log2 of the lanes one row takes
 };
 
 template <int DT>
@@ -653,14 +655,16 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
     }
 }
 
-// Rows of at most 64 whole vectors, every tensor on one 16-byte grid.  One wavefront per row
-// would leave most lanes idle and walk the batch one short row at a time, so a wavefront takes
-// 64 / G batch entries of its channel at once, G = 8, 16, 32 or 64 lanes each: lane (r, v) owns
-// vector v of entry r, x's halo comes from the previous lane (vector 0: zeros or initial_states),
-// g's from the next lane (last vector: zeros), and an item is one load of x, one of dout and one
-// store of dx per lane.  Formulas, operation order and the reduction at the end are those of the
-// kernels above, so results do not depend on which kernel a shape takes.
-template <int DT, int W>
+// Rows of at most 64 vectors.  One wavefront per row would leave most lanes idle and walk the
+// batch one short row at a time, so a wavefront takes 64 / G batch entries of its channel at once,
+// G = 1, 2, 4 ... 64 lanes each: lane (r, v) owns vector v of entry r, x's halo comes from the
+// previous lane (vector 0: zeros or initial_states), g's from the next lane (last vector: zeros),
+// and an item is one load of x, one of dout and one store of dx per lane.  Formulas, operation
+// order and the reduction at the end are those of the kernels above.
+// ALIGNED: rows of whole vectors, every tensor on one 16-byte grid.  ALIGNED = false: rows of any
+// length (down to 1) anywhere in memory, the same lanes, with a lane's up to VEC positions read
+// and written element by element (positions past the row's end read as zero).
+template <int DT, int W, bool ALIGNED>
 __global__ void __launch_bounds__(kBlock)
 bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__restrict__ ws) {
     using E = Elem<DT>;
@@ -672,7 +676,8 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
     if (wid >= (uint32_t)p.dim * (uint32_t)g.n_parts) return;     // whole wave leaves together
     const int part = (int)(wid % (uint32_t)g.n_parts);
     const int c = (int)(wid / (uint32_t)g.n_parts);
-    const int n_vecs = p.seqlen / VEC;
+    const int L = p.seqlen;
+    const int n_vecs = (L + VEC - 1) / VEC;
     const int v = lane & ((1 << g.lanes_log2) - 1);
     const int r = lane >> g.lanes_log2;
     const int rows_per_item = kWave >> g.lanes_log2;
@@ -702,10 +707,27 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
         const int64_t drow = (int64_t)b * p.dout_stride_b + (int64_t)c * p.dout_stride_c;
         const int64_t dxrow = (int64_t)b * p.dx_stride_b + (int64_t)c * p.dx_stride_c;
 
-        u32x4 rx = u32x4{0u, 0u, 0u, 0u}, rd = u32x4{0u, 0u, 0u, 0u};
-        if (mine) {
-            rx = ld_vec_nt<DT>(p.x, xrow + (int64_t)v * VEC);
-            rd = ld_vec_nt<DT>(p.dout, drow + (int64_t)v * VEC);
+        float xf[VEC], gf[VEC];
+        if (ALIGNED) {
+            u32x4 rx = u32x4{0u, 0u, 0u, 0u}, rd = u32x4{0u, 0u, 0u, 0u};
+            if (mine) {
+                rx = ld_vec_nt<DT>(p.x, xrow + (int64_t)v * VEC);
+                rd = ld_vec_nt<DT>(p.dout, drow + (int64_t)v * VEC);
+            }
+            E::unpack(rx, xf);
+            E::unpack(rd, gf);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xf[e] = gf[e] = 0.f;
+            if (mine) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if (v * VEC + e < L) {
+                        xf[e] = ld_elem<DT>(p.x, xrow + v * VEC + e);
+                        gf[e] = ld_elem<DT>(p.dout, drow + v * VEC + e);
+                    }
+                }
+            }
         }
         float halo[W - 1];
 #pragma unroll
@@ -716,9 +738,6 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
                 halo[i] = ld_elem<DT>(p.initial_states, (int64_t)b * p.init_stride_b + (int64_t)c * p.init_stride_c +
                                                             (int64_t)i * p.init_stride_l);
         }
-        float xf[VEC], gf[VEC];
-        E::unpack(rx, xf);
-        E::unpack(rd, gf);
 
         // xx[i] = xpad at position v*VEC-(W-1)+i
         float xx[VEC + W - 1];
@@ -758,15 +777,31 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
             for (int k = 0; k < W; ++k) a = fmaf(wv[W - 1 - k], gg[e + k], a);
             dxv[e] = a;
         }
-        // The row's last W-1 positions (all in its last vector) take dfinal_states.
-        if (p.dfinal_states != nullptr && mine && v == n_vecs - 1) {
+        // The row's last W-1 positions take dfinal_states (whole vectors: all in the last one).
+        if (ALIGNED) {
+            if (p.dfinal_states != nullptr && mine && v == n_vecs - 1) {
 #pragma unroll
-            for (int i = 0; i < W - 1; ++i)
-                dxv[VEC - (W - 1) + i] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
-                                                                           (int64_t)c * p.dfinal_stride_c +
-                                                                           (int64_t)i * p.dfinal_stride_l);
+                for (int i = 0; i < W - 1; ++i)
+                    dxv[VEC - (W - 1) + i] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
+                                                                               (int64_t)c * p.dfinal_stride_c +
+                                                                               (int64_t)i * p.dfinal_stride_l);
+            }
+            if (mine) st_vec_nt<DT>(p.dx, dxrow + (int64_t)v * VEC, E::pack(dxv));
+        } else if (mine) {
+            if (p.dfinal_states != nullptr && (v + 1) * VEC > L - (W - 1)) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const int t = v * VEC + e;
+                    if (t >= L - (W - 1) && t < L)
+                        dxv[e] += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b +
+                                                                   (int64_t)c * p.dfinal_stride_c +
+                                                                   (int64_t)(t - (L - (W - 1))) * p.dfinal_stride_l);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                if (v * VEC + e < L) st_elem<DT>(p.dx, dxrow + v * VEC + e, dxv[e]);
         }
-        if (mine) st_vec_nt<DT>(p.dx, dxrow + (int64_t)v * VEC, E::pack(dxv));
 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -776,7 +811,8 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
         }
 
         // dinitial_states[b, c, i]: the expression of dx at position i-(W-1) < 0, by the lane that
-        // owns vector 0 (a row of whole vectors is never shorter than W-1).
+        // owns vector 0; where the row is shorter than W-1, final_states[i-L] was a copy of
+        // initial_states[i], so its gradient lands here.
         if (p.dinitial_states != nullptr && mine && v == 0) {
 #pragma unroll
             for (int i = 0; i < W - 1; ++i) {
@@ -786,6 +822,9 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
                     const int t = i - (W - 1) + k;
                     a = fmaf(wv[W - 1 - k], t >= 0 ? gf[t] : 0.f, a);
                 }
+                if (!ALIGNED && p.dfinal_states != nullptr && i >= L)
+                    a += ld_elem<DT>(p.dfinal_states, (int64_t)b * p.dfinal_stride_b + (int64_t)c * p.dfinal_stride_c +
+                                                          (int64_t)(i - L) * p.dfinal_stride_l);
                 st_elem<DT>(p.dinitial_states, (int64_t)b * p.dinit_stride_b + (int64_t)c * p.dinit_stride_c +
                                                    (int64_t)i * p.dinit_stride_l, a);
             }
@@ -846,13 +885,16 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     // Short rows of whole vectors with every tensor on one grid: several batch entries to a
     // wavefront, an item is a group of them.  (16, 5376, 128) bf16 57.2 -> 16.0 us, fp32 43.0 -> 25.0 us;
     // (4, 5376, 256) bf16 18.2 -> 10.3 us.
-    const int64_t n_vecs = p.seqlen / vec;
-    if (on_grid && n_vecs >= 1 && n_vecs <= kWave &&
-        rows_share_grid(p.x, p.x_stride_b, p.x_stride_c, p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
-        rows_share_grid(p.x, p.x_stride_b, p.x_stride_c, p.dx, p.dx_stride_b, p.dx_stride_c, vec)) {
-        g.lanes_log2 = n_vecs <= 8 ? 3 : n_vecs <= 16 ? 4 : n_vecs <= 32 ? 5 : 6;
+    // Rows that are not whole vectors on one grid take the same lanes with element accesses:
+    // (16, 5376, 100) bf16 107 -> 39 us, (64, 2048, 60) 165 -> 36 us, (256, 5376, 4) 1514 -> 73 us.
+    const int64_t n_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
+    if (n_vecs <= kWave) {
+        const bool aligned = on_grid &&
+            rows_share_grid(p.x, p.x_stride_b, p.x_stride_c, p.dout, p.dout_stride_b, p.dout_stride_c, vec) &&
+            rows_share_grid(p.x, p.x_stride_b, p.x_stride_c, p.dx, p.dx_stride_b, p.dx_stride_c, vec);
+        while ((1 << g.lanes_log2) < n_vecs) ++g.lanes_log2;
         const int64_t per_item = kWave >> g.lanes_log2;
-        g.streaming = 3;
+        g.streaming = aligned ? 3 : 4;
         g.vecs_per_seg = kWave;
         g.n_segs = 1;
         g.n_items = (int32_t)((p.batch + per_item - 1) / per_item);
@@ -877,9 +919,17 @@ int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStr
     const uint32_t blocks = (uint32_t)((waves + (kBlock / kWave) - 1) / (kBlock / kWave));
     if (g.streaming == 3) {                           // short rows, several batch entries to a wavefront
         switch (p.width) {
-            case 2: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            case 3: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            default: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 2: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 2, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 3, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 4, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        }
+        return launch_status();
+    }
+    if (g.streaming == 4) {                           // the same, rows of any length anywhere in memory
+        switch (p.width) {
+            case 2: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 2, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 3, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 4, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         }
         return launch_status();
     }

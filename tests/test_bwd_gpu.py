@@ -89,7 +89,7 @@ def test_bwd_channel_first_short_rows(pkg, gpu_device, seqlen, dtype):
     """Channel-first rows of at most 64 whole 16-byte vectors: several batch entries share a
     wavefront.  A batch that does not fill the last group, every vector-count class, all state
     gradients; dx and dinitial_states must also equal, bit for bit, what the same data gives
-    when it sits one element off the 16-byte grid (which takes the walking kernel)."""
+    when it sits one element off the 16-byte grid (element accesses instead of vectors)."""
     dev = gpu_device
     batch, dim, width = 5, 24, 2 + seqlen % 3
     g = gen(2000 + seqlen)
@@ -113,6 +113,28 @@ def test_bwd_channel_first_short_rows(pkg, gpu_device, seqlen, dtype):
     # no states, no bias, no activation
     got = run_gpu(pkg, dev, x, w, None, dout)
     check(got, orc.bwd(x, w, None, dout), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seqlen", [1, 2, 3, 5, 7, 9, 60, 100, 255, 500])
+def test_bwd_channel_first_short_rows_of_any_length(pkg, gpu_device, seqlen, dtype):
+    """Channel-first rows of at most 64 vectors that are not whole vectors share wavefronts too,
+    down to one lane per batch entry.  All state gradients: in a row shorter than width-1 part of
+    dfinal_states lands in dinitial_states (csrc/causal_conv1d_bwd.cu:535-561)."""
+    dev = gpu_device
+    batch, dim = 67, 24                                # more entries than one wavefront takes at once
+    for width in (2, 3, 4):
+        g = gen(4000 + seqlen * 4 + width)
+        x = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+        dout = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+        w, b = make_wb(dim, width, True, g)
+        init = make_states(batch, dim, width - 1, dtype, g)
+        dfin = make_states(batch, dim, width - 1, dtype, g)
+        ref = orc.bwd(x, w, b, dout, initial_states=init, dfinal_states=dfin, activation="silu")
+        got = run_gpu(pkg, dev, x, w, b, dout, init=init, dfin=dfin, act="silu")
+        check(got, ref, dtype)
+        got = run_gpu(pkg, dev, x, w, None, dout)
+        check(got, orc.bwd(x, w, None, dout), dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -89,6 +89,30 @@ def test_fwd_channel_first_short_rows(pkg, gpu_device, seqlen, dtype):
     assert_close(plain, orc.fwd(xs, w, None), dtype, "no bias, no activation, no states")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seqlen", [1, 2, 3, 5, 7, 9, 60, 100, 255, 500])
+def test_fwd_channel_first_short_rows_of_any_length(pkg, gpu_device, seqlen, dtype):
+    """Channel-first rows of at most 64 vectors that are not whole vectors (a contiguous tensor
+    whose seqlen is no multiple of 16 bytes) share wavefronts too, down to one lane per row; rows
+    shorter than width-1 take part of final_states from initial_states (or zeros)."""
+    dev = gpu_device
+    batch, dim = 3, 40
+    for width in (2, 3, 4):
+        g = gen(3000 + seqlen * 4 + width)
+        x = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+        w, b = make_wb(dim, width, True, g)
+        init = make_states(batch, dim, width - 1, dtype, g)
+        ref, ref_fin = orc.fwd(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+        got, got_fin = pkg.causal_conv1d_fn(x.to(dev), w.to(dev), b.to(dev), initial_states=init.to(dev),
+                                            return_final_states=True, activation="silu")
+        assert_close(got, ref, dtype, "out")
+        assert torch.equal(got_fin.cpu(), ref_fin)
+        ref, ref_fin = orc.fwd(x, w, None, return_final_states=True)
+        got, got_fin = pkg.causal_conv1d_fn(x.to(dev), w.to(dev), None, return_final_states=True)
+        assert_close(got, ref, dtype, "no bias, no activation, no initial states")
+        assert torch.equal(got_fin.cpu(), ref_fin)
+
+
 @pytest.mark.parametrize("pad", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("dim,seqlen,width,has_bias,silu", [
