@@ -94,9 +94,11 @@ def test_fwd_channel_first_short_rows(pkg, gpu_device, seqlen, dtype):
 def test_fwd_channel_first_short_rows_of_any_length(pkg, gpu_device, seqlen, dtype):
     """Channel-first rows of at most 64 vectors that are not whole vectors (a contiguous tensor
     whose seqlen is no multiple of 16 bytes) share wavefronts too, down to one lane per row; rows
-    shorter than width-1 take part of final_states from initial_states (or zeros)."""
+    shorter than width-1 take part of final_states from initial_states (or zeros).  Contiguous
+    tensors with rows of at least one vector are walked as one flat array of whole vectors, a
+    vector spanning two rows; slices of a wider tensor take element accesses."""
     dev = gpu_device
-    batch, dim = 3, 40
+    batch, dim = 3, 41                                 # batch * dim * seqlen is no whole number of vectors either
     for width in (2, 3, 4):
         g = gen(3000 + seqlen * 4 + width)
         x = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
@@ -111,6 +113,17 @@ def test_fwd_channel_first_short_rows_of_any_length(pkg, gpu_device, seqlen, dty
         got, got_fin = pkg.causal_conv1d_fn(x.to(dev), w.to(dev), None, return_final_states=True)
         assert_close(got, ref, dtype, "no bias, no activation, no initial states")
         assert torch.equal(got_fin.cpu(), ref_fin)
+        wide = torch.zeros(batch, dim, seqlen + 3, dtype=dtype)
+        wide[:, :, 2:2 + seqlen] = x
+        ref, ref_fin = orc.fwd(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+        sliced, sliced_fin = pkg.causal_conv1d_fn(wide.to(dev)[:, :, 2:2 + seqlen], w.to(dev), b.to(dev),
+                                                  initial_states=init.to(dev), return_final_states=True,
+                                                  activation="silu")
+        assert_close(sliced, ref, dtype, "out of a slice")
+        if seqlen * x.element_size() <= 1024:          # both are short rows: one arithmetic, two access patterns
+            assert torch.equal(sliced, pkg.causal_conv1d_fn(x.to(dev), w.to(dev), b.to(dev),
+                                                            initial_states=init.to(dev), activation="silu"))
+        assert torch.equal(sliced_fin.cpu(), ref_fin)
 
 
 @pytest.mark.parametrize("pad", [False, True])
