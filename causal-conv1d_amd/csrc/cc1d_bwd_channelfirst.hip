@@ -873,12 +873,6 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int64_t max_parts = (int64_t)p.batch * max_steps;
     if (parts > max_parts) parts = max_parts;
     if (parts < 1) parts = 1;
-    // Split rows into segments only if there are fewer rows per channel than slices.
-    int64_t n_segs = (parts + p.batch - 1) / p.batch;
-    int64_t steps_per_seg = (max_steps + n_segs - 1) / n_segs;
-    if (streaming) steps_per_seg = (steps_per_seg + 1) / 2 * 2;    // whole step pairs
-    int64_t vps = steps_per_seg * kWave;
-    n_segs = (max_vecs + vps - 1) / vps;
     BwdCfGeom g;
     const bool on_grid = aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 && p.seqlen % vec == 0;
     g.lanes_log2 = 0;
@@ -903,6 +897,22 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
         g.n_parts = (g.n_items + g.items_per_part - 1) / g.items_per_part;
         return g;
     }
+    // The chip holds about 4096 of these wavefronts at once.  A launch of 1 to 1.5 times that many
+    // long-lived ones ends with the chip mostly idle while the last few finish, so it is cut finer
+    // instead, down to eight steps of work per wavefront: (32, 1536, 2048) bf16 126 -> 107 us,
+    // (64, 768, 1024) 69 -> 65 us, (8, 5376, 2048) fp32 205 -> 175 us, (1, 5376, 131072) bf16 875 -> 690 us;
+    // other wave counts measured best as they are.
+    if (tunables().bwd_cf_parts <= 0 && p.dim * parts > 4096 && 2 * p.dim * parts < 3 * 4096) {
+        int64_t finer = p.batch * max_steps / 8;
+        if (finer > 64) finer = 64;
+        if (finer > parts) parts = finer;
+    }
+    // Split rows into segments only if there are fewer rows per channel than slices.
+    int64_t n_segs = (parts + p.batch - 1) / p.batch;
+    int64_t steps_per_seg = (max_steps + n_segs - 1) / n_segs;
+    if (streaming) steps_per_seg = (steps_per_seg + 1) / 2 * 2;    // whole step pairs
+    int64_t vps = steps_per_seg * kWave;
+    n_segs = (max_vecs + vps - 1) / vps;
     g.streaming = !streaming ? 0 : on_grid ? 1 : 2;
     g.vecs_per_seg = (int32_t)vps;
     g.n_segs = (int32_t)n_segs;
