@@ -82,7 +82,6 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     if (wave >= g.total) return;
     const uint32_t col = (wave % g.waves_per_row) * (uint32_t)kWave + (threadIdx.x & (kWave - 1));
     const uint32_t rb = wave / g.waves_per_row;
-    if (col >= (uint32_t)g.n_colgroups) return;       // no cross-lane traffic below
     const int run = (int)(rb % (uint32_t)g.n_runs);
     const int b = (int)(rb / (uint32_t)g.n_runs);
     const int c0 = (int)col * CH;
@@ -90,6 +89,45 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     const int T = g.rows_per_run;                     // multiple of 2*U
     const int t0 = run * T;                           // < L by construction of n_runs
     const int last = L - 1 - t0;                      // last valid row of this run, run-relative
+
+    // With seq_idx the walk computes every row as if no sub-sequence boundary were near (no
+    // branch, no ids in the hot loop); the groups of U rows whose rows or window are not all of
+    // one non-negative id are redone with masked taps after the walk.  Which groups those are is
+    // found here, with all 64 lanes, a row per lane: lane i holds row i-(W-1) of a stretch of
+    // whole groups and flags it when its id differs from the row before or is negative (rows in
+    // front of the sequence count as id -1 when initial_states are given, as zeros, which no
+    // mask changes, otherwise); group k is redone when a flag falls into its rows or the W-2
+    // rows before them.  Where more than half of the groups are (sub-sequences of a few tokens),
+    // the walk is skipped and the masked pass takes the whole run.
+    uint32_t redo = 0;
+    bool dense = false;
+    if (HAS_SEQ) {
+        const int n_groups = T / U;
+        if (n_groups > 32) {
+            dense = true;
+        } else {
+            constexpr int kStretch = (kWave - (W - 1)) / U;            // groups per look
+            const int32_t *ids = seq_idx + (int64_t)b * L;
+            const int lane = threadIdx.x & (kWave - 1);
+            const bool init = p.initial_states != nullptr;
+            for (int k0 = 0; k0 < n_groups; k0 += kStretch) {
+                const int t_lane = t0 + k0 * U + lane - (W - 1);       // row of this lane
+                const int t = t_lane > L - 1 ? L - 1 : t_lane;
+                const int id = ids[t > 0 ? t : 0];
+                const int id_prev = ids[t > 1 ? t - 1 : 0];
+                const bool flag = t_lane > L - 1 ? false
+                                : t >= 0 ? (id < 0 || (t > 0 ? id != id_prev : init)) : init;
+                const uint64_t flags = __ballot(flag);
+                for (int k = 0; k < kStretch && k0 + k < n_groups; ++k)
+                    if ((flags >> (k * U + 1)) & ((1ull << (U + W - 2)) - 1)) redo |= 1u << (k0 + k);
+            }
+            int live = last / U + 1;                                   // groups with rows inside the sequence
+            live = live > n_groups ? n_groups : live;
+            redo &= live >= 32 ? ~0u : (1u << live) - 1u;
+            dense = 2 * __builtin_popcount(redo) > live;
+        }
+    }
+    if (col >= (uint32_t)g.n_colgroups) return;       // no cross-lane traffic below
 
     // Packed taps are only requested here: everything the run starts with is in flight before
     // the first value is touched (prepare() finishes them).
@@ -123,14 +161,11 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     char *orun = reinterpret_cast<char *>(reinterpret_cast<T_ *>(p.out) + ooff + (int64_t)t0 * p.out_stride_l);
     const uint32_t xs = (uint32_t)p.x_stride_l * (uint32_t)sizeof(T_);
     const uint32_t os = (uint32_t)p.out_stride_l * (uint32_t)sizeof(T_);
-    // seq_idx is a kernel argument of its own, marked as not aliasing anything the kernel
-    // writes: its loads, at wave-uniform addresses, then go through the scalar cache.
     const int32_t *seq = HAS_SEQ ? seq_idx + (int64_t)b * L + t0 : nullptr;
 
     // Sliding window: xw[i] holds row t-(W-1)+i while row t is being produced.  The halo
     // rows are requested here and unpacked by prepare().
     float xw[W - 1][CH];
-    int sqw[W - 1];
     raw_t halo[W - 1];
 #pragma unroll
     for (int i = 0; i < W - 1; ++i) {
@@ -142,10 +177,6 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
             halo[i] = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
                                              p.init_stride_l, b, c0, t + (W - 1));
         }
-        // Rows in front of the sequence hold zeros unless initial_states are given; with
-        // zeros a mask changes nothing, so they take the first row's id and do not make
-        // the first group look like a boundary.
-        sqw[i] = !HAS_SEQ ? 0 : t >= 0 ? seq[i - (W - 1)] : p.initial_states != nullptr ? -1 : seq[-t0];
     }
     auto prepare = [&]() {
         scale_taps();
@@ -160,36 +191,16 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     // past its end re-read the last valid row and their stores are suppressed.
     // STREAM: non-temporal loads; the last rows of a run are read with the normal policy
     // because the following run needs them again as its halo.
-    auto load_group = [&](auto checked, auto stream, int i0, raw_t (&raw)[U], int (&sq)[U]) {
+    auto load_group = [&](auto checked, auto stream, int i0, raw_t (&raw)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
             const raw_t *src = reinterpret_cast<const raw_t *>(xrun + (uint32_t)i * xs);
             raw[u] = decltype(stream)::value ? __builtin_nontemporal_load(src) : *src;
-            sq[u] = HAS_SEQ ? seq[i] : 0;             // wave-uniform address: a scalar load
         }
     };
 
-    // With seq_idx the walk computes every row as if no sub-sequence boundary were near
-    // (no branch in the hot loop) and only records, per wavefront, the span of row groups whose
-    // rows or window are not all of one non-negative id.  Those few rows are redone with
-    // masked taps after the walk.
-    int redo_lo = T, redo_hi = 0;
-    auto compute_group = [&](auto checked, int i0, const raw_t (&raw)[U], const int (&sq)[U]) {
-        if (HAS_SEQ) {
-            // The ids sit in scalar registers and the bookkeeping runs on the scalar unit.
-            int id[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) id[u] = sq[u];
-            uint32_t lo = (uint32_t)id[0], hi = (uint32_t)id[0];
-#pragma unroll
-            for (int u = 1; u < U; ++u) { lo = min(lo, (uint32_t)id[u]); hi = max(hi, (uint32_t)id[u]); }
-#pragma unroll
-            for (int k = 0; k < W - 1; ++k) { lo = min(lo, (uint32_t)sqw[k]); hi = max(hi, (uint32_t)sqw[k]); }
-            if (lo != hi || (int)hi < 0) { redo_lo = min(redo_lo, i0); redo_hi = max(redo_hi, i0 + U); }
-#pragma unroll
-            for (int k = 0; k < W - 1; ++k) sqw[k] = id[U - (W - 1) + k];
-        }
+    auto compute_group = [&](auto checked, int i0, const raw_t (&raw)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float xv[CH], acc[CH];
@@ -217,8 +228,10 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     using Yes = std::integral_constant<bool, true>;
     static_assert(U >= W - 1, "a group must cover the window");
     raw_t ra[U], rb_[U];
-    int sa[U], sb[U];
-    if (last >= T - 1) {
+    if (dense) {
+        // Most groups would be redone: skip the walk, the masked pass below takes the whole run.
+        prepare();
+    } else if (last >= T - 1) {
         // Two register sets in ping-pong: while one group of U rows is computed and stored,
         // the next two groups' loads are in flight, and nothing is copied at the loop edge
         // (a copy would make the compiler wait for every outstanding access).  The first
@@ -226,45 +239,45 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         // state its back edge leaves (stores A, loads A, stores B, loads B pending), which
         // keeps the compiler's wait counts exact, and no load sits behind an exit test.
         if (T > 2 * U) {
-            load_group(No{}, Yes{}, 0, ra, sa);
-            load_group(No{}, Yes{}, U, rb_, sb);
+            load_group(No{}, Yes{}, 0, ra);
+            load_group(No{}, Yes{}, U, rb_);
             prepare();
-            compute_group(No{}, 0, ra, sa);
+            compute_group(No{}, 0, ra);
             int i = 2 * U;
             if (T > 4 * U) {
-                load_group(No{}, Yes{}, 2 * U, ra, sa);
-                compute_group(No{}, U, rb_, sb);
-                load_group(No{}, Yes{}, 3 * U, rb_, sb);
+                load_group(No{}, Yes{}, 2 * U, ra);
+                compute_group(No{}, U, rb_);
+                load_group(No{}, Yes{}, 3 * U, rb_);
 #pragma clang loop unroll(disable)
                 for (; i + 4 * U < T; i += 2 * U) {
-                    compute_group(No{}, i, ra, sa);
-                    load_group(No{}, Yes{}, i + 2 * U, ra, sa);
-                    compute_group(No{}, i + U, rb_, sb);
-                    load_group(No{}, Yes{}, i + 3 * U, rb_, sb);
+                    compute_group(No{}, i, ra);
+                    load_group(No{}, Yes{}, i + 2 * U, ra);
+                    compute_group(No{}, i + U, rb_);
+                    load_group(No{}, Yes{}, i + 3 * U, rb_);
                 }
-                compute_group(No{}, i, ra, sa);
-                load_group(No{}, Yes{}, i + 2 * U, ra, sa);
-                compute_group(No{}, i + U, rb_, sb);
+                compute_group(No{}, i, ra);
+                load_group(No{}, Yes{}, i + 2 * U, ra);
+                compute_group(No{}, i + U, rb_);
                 i += 2 * U;
             } else {
-                load_group(No{}, Yes{}, 2 * U, ra, sa);
-                compute_group(No{}, U, rb_, sb);
+                load_group(No{}, Yes{}, 2 * U, ra);
+                compute_group(No{}, U, rb_);
             }
-            load_group(No{}, No{}, i + U, rb_, sb);   // the run's last rows: keep them cached
-            compute_group(No{}, i, ra, sa);
-            compute_group(No{}, i + U, rb_, sb);
+            load_group(No{}, No{}, i + U, rb_);   // the run's last rows: keep them cached
+            compute_group(No{}, i, ra);
+            compute_group(No{}, i + U, rb_);
         } else {
-            load_group(No{}, Yes{}, 0, ra, sa);
-            load_group(No{}, No{}, U, rb_, sb);
+            load_group(No{}, Yes{}, 0, ra);
+            load_group(No{}, No{}, U, rb_);
             prepare();
-            compute_group(No{}, 0, ra, sa);
-            compute_group(No{}, U, rb_, sb);
+            compute_group(No{}, 0, ra);
+            compute_group(No{}, U, rb_);
         }
     } else {
         prepare();
         for (int i = 0; i <= last; i += U) {
-            load_group(Yes{}, No{}, i, ra, sa);
-            compute_group(Yes{}, i, ra, sa);
+            load_group(Yes{}, No{}, i, ra);
+            compute_group(Yes{}, i, ra);
         }
     }
 
@@ -274,8 +287,10 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         // zero.  All U+W-1 rows and ids a group needs are requested at once, straight from
         // memory (they were streamed moments ago), with no branch between the loads; the
         // results overwrite what the walk stored for these rows.
+        const int live_rows = last + 1 < T ? last + 1 : T;
 #pragma clang loop unroll(disable)
-        for (int i0 = redo_lo; i0 < redo_hi; i0 += U) {
+        for (int i0 = 0; i0 < live_rows; i0 += U) {
+            if (!dense && !((redo >> (i0 / U)) & 1u)) continue;
             float xr[U + W - 1][CH];
             int sr[U + W - 1];
 #pragma unroll

@@ -148,6 +148,30 @@ def test_fwd_seq_idx_matches_per_segment_oracle(pkg, gpu_device, dim, seqlen, wi
         assert torch.all(got.cpu()[(seq < 0).unsqueeze(1).expand_as(got)] == 0), "padding must be exact zeros"
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim,seqlen,width,every", [(64, 333, 4, 1), (64, 1000, 3, 3), (264, 517, 4, 5), (264, 2048, 2, 2),
+                                                    (4128, 300, 4, 4), (128, 4096, 4, 16)])
+def test_fwd_seq_idx_with_sub_sequences_of_a_few_tokens(pkg, gpu_device, dim, seqlen, width, every, dtype):
+    """Boundaries every few rows (and a padded tail): most groups of a run hold one, which takes
+    the masked pass without the walk; boundaries every 16 rows mark about half of them."""
+    g = gen(seqlen + dim + every)
+    x = make_x(2, dim, seqlen, dtype, True, g)
+    w, b = make_wb(dim, width, True, g)
+    rows = []
+    for _ in range(2):
+        cuts = torch.zeros(seqlen, dtype=torch.int32)
+        cuts[torch.randperm(seqlen - 1, generator=g)[:seqlen // every] + 1] = 1
+        ids = torch.cumsum(cuts, 0).to(torch.int32)
+        if every % 2 == 1:
+            ids[seqlen - int(torch.randint(1, seqlen // 3, (1,), generator=g)):] = -1   # padded tail
+        rows.append(ids)
+    seq = torch.stack(rows)
+    ref = orc.fwd_seq_idx(x, w, b, seq, activation="silu")
+    got = pkg.causal_conv1d_fn(to_dev_like(x, gpu_device), w.to(gpu_device), b.to(gpu_device),
+                               seq_idx=seq.to(gpu_device), activation="silu")
+    assert_close(got, ref, dtype, "out")
+
+
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("channel_last", [False, True])
