@@ -90,6 +90,14 @@ fwd_channelfirst_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
         for (int w = 0; w < W; ++w)
             wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
         bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+        // The arithmetic of the other kernels, bit for bit: taps and bias carry the factor
+        // -log2(e) where the activation takes the sums as its exponent (see silu_from_scaled).
+        const bool scaled = silu_on && !PRECISE;
+        if (scaled) {
+            bias_v *= kSiluPrescale;
+#pragma unroll
+            for (int w = 0; w < W; ++w) wv[w] *= kSiluPrescale;
+        }
 
         // Halo of the segment's first vector, wave-uniform.
         float carry[W - 1];
@@ -132,7 +140,7 @@ fwd_channelfirst_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
                 float a = bias_v;
 #pragma unroll
                 for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
-                acc[e] = silu_on ? silu<PRECISE>(a) : a;
+                acc[e] = scaled ? silu_from_scaled(a) : silu_on ? silu<PRECISE>(a) : a;
             }
 
             const int j = j0 + lane;
