@@ -16,7 +16,7 @@
 // initial_states / final_states are supported (the reference refuses them for this
 // layout, csrc/causal_conv1d.cpp:213,228).
 //
-// Three kernels share this design.  The streaming kernel takes every launch in which the rows
+// Four kernels share this design.  The streaming kernel takes every launch in which the rows
 // of out lie on the same 16-byte grid as the rows of x (same shape and strides, as
 // empty_like gives): whole 64-vector steps run without bounds checks in two register sets in
 // ping-pong, which keep the loads of the next two groups in flight while a group is computed
