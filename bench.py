@@ -392,6 +392,18 @@ def main():
         for ln in open(traffic_file):
             if ln.startswith("traffic_bytes_per_launch:"):
                 line["roofline"]["traffic"] = int(float(ln.split(":")[1]))
+    if not args.no_others:
+        # The same call over six rotating sets of x and out (2.1 GB): every launch then meets cold
+        # address translations and caches, as the layers of a model do; next to it PyTorch's
+        # elementwise add over the same sets (the same bytes in, the same bytes out).
+        sets = [(x, out)] + [(torch.randn_like(x), torch.empty_like(x)) for _ in range(5)]
+        rot_us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(sets[i % 6][0], w, b, seq, None, sets[i % 6][1], None, True),
+                             args.steps, args.warmup)
+        add_us, _ = time_gpu(lambda i: torch.add(sets[i % 6][0], 1.0, out=sets[i % 6][1]), args.steps, args.warmup)
+        line["config"].update({"us_per_call_rotated": round(rot_us, 3), "rotated_sets": 6,
+                               "GBps_rotated": round(gbs(n_bytes, rot_us), 1),
+                               "us_torch_add_rotated": round(add_us, 3)})
+        del sets
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg_cpu, n_bytes, gpu_out_host)
     del cfg, x, out

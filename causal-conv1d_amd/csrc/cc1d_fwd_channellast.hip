@@ -22,6 +22,10 @@
 
 #include "cc1d_varlen_gather.hpp"
 
+// 1: rows that no later run needs are loaded non-temporally; 0: every load takes the normal policy.
+#ifndef CC1D_FWD_CL_STREAM_LOADS
+#define CC1D_FWD_CL_STREAM_LOADS 1
+#endif
 // Rows per register set; two sets are in flight per lane.
 #ifndef CC1D_FWD_CL_UNROLL
 #define CC1D_FWD_CL_UNROLL 8
@@ -43,7 +47,19 @@
 namespace cc1d {
 namespace {
 
-constexpr int kXcds = 8;
+#ifndef CC1D_FWD_CL_STREAM_STORES
+#define CC1D_FWD_CL_STREAM_STORES 1
+#endif
+template <typename V>
+__device__ __forceinline__ void store_row(const V &v, V *dst) {
+    if (CC1D_FWD_CL_STREAM_STORES) __builtin_nontemporal_store(v, dst);
+    else *dst = v;
+}
+
+#ifndef CC1D_FWD_CL_XCDS
+#define CC1D_FWD_CL_XCDS 8
+#endif
+constexpr int kXcds = CC1D_FWD_CL_XCDS;
 
 struct FwdClGeom {
     int32_t rows_per_run;     // T, a multiple of twice the unroll factor
@@ -196,7 +212,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         for (int u = 0; u < U; ++u) {
             const int i = (!decltype(checked)::value || (i0 + u) < last) ? (i0 + u) : last;
             const raw_t *src = reinterpret_cast<const raw_t *>(xrun + (uint32_t)i * xs);
-            raw[u] = decltype(stream)::value ? __builtin_nontemporal_load(src) : *src;
+            raw[u] = (decltype(stream)::value && CC1D_FWD_CL_STREAM_LOADS) ? __builtin_nontemporal_load(src) : *src;
         }
     };
 
@@ -214,7 +230,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
                 acc[j] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
             }
             if (!decltype(checked)::value || i0 + u <= last)
-                __builtin_nontemporal_store(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
+                store_row(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
 #pragma unroll
             for (int k = 0; k < W - 2; ++k)
 #pragma unroll
@@ -318,7 +334,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
                     acc[j] = cur < 0 ? 0.f : a;
                 }
                 if (i0 + u <= last)
-                    __builtin_nontemporal_store(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
+                    store_row(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
             }
         }
     }
