@@ -14,9 +14,10 @@
 // ceil(dim / (64 CH)) wavefronts, the last one partly idle when dim is not a multiple of
 // 64 CH.  Wavefronts are numbered (batch, run, column block) with the column block
 // fastest, and workgroups are renumbered so that each of the 8 XCDs (hardware hands
-// workgroups to XCDs round-robin) walks a contiguous slice of that order: the run that
-// follows another along seqlen then executes on the same XCD, close in time, and its halo rows are found in that XCD's L2 instead of being fetched from
-// HBM twice.  For the same reason the halo rows and the last rows of a run are accessed
+// workgroups to XCDs round-robin) walks chunks of consecutive runs of that order (8 runs, the
+// XCDs side by side on 8 neighbouring chunks): the run that follows another along seqlen then
+// executes on the same XCD, close in time, and its halo rows are found in that XCD's L2
+// instead of being fetched from HBM twice.  For the same reason the halo rows and the last rows of a run are accessed
 // with the normal cache policy while everything else streams through (non-temporal).
 #include <type_traits>
 
@@ -68,6 +69,7 @@ struct FwdClGeom {
     uint32_t waves_per_row;   // ceil(n_colgroups / 64): wavefronts side by side on one row
     uint32_t total;           // batch * n_runs * waves_per_row wavefronts
     uint32_t blocks_per_xcd;  // grid size / 8
+    uint32_t blocks_per_chunk; // workgroups an XCD takes in a row before the next XCD's (0: its whole slice)
 };
 
 // WM: how the taps are read.  1: packed (dim, W) fp32, 2: packed in x's own 16-bit type (both
@@ -90,7 +92,10 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         return;
     }
     // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
-    const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
+    const uint32_t xcd = blockIdx.x % kXcds, nth = blockIdx.x / kXcds;
+    const uint32_t block = g.blocks_per_chunk == 0
+                               ? xcd * g.blocks_per_xcd + nth
+                               : ((nth / g.blocks_per_chunk) * kXcds + xcd) * g.blocks_per_chunk + nth % g.blocks_per_chunk;
     // A wavefront never straddles two runs: its batch index, run and row range are scalars,
     // and so are the sub-sequence ids it reads.
     const uint32_t wave = block * (uint32_t)(kBlock / kWave) +
@@ -445,7 +450,26 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     if (total * kWave >= ((int64_t)1 << 31) - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
     g.total = (uint32_t)total;
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
+    // Workgroup order: an XCD takes chunks of `chunk_runs` consecutive runs (all their column
+    // blocks), the 8 XCDs take 8 neighbouring chunks at a time.
+    // Against one contiguous slice of the launch per XCD (8 streams far apart in memory, each with
+    // its own address translations to fetch), chunks of 8 runs measured, warm / on rotating buffers
+    // that do not fit the translation caches: (8, 5376, 2048) bf16 55.6 / 65.1 -> 55.8 / 63.9 us,
+    // (4, 4096, 4096) 43.9 / 51.8 -> 43.5 / 50.0 us, (16, 2048, 2048) 46.3 / 56.2 -> 43.7 / 49.5 us.  Only the
+    // first run of a chunk finds its halo rows in another XCD's L2.  Launches of fewer than eight
+    // chunks per XCD take chunks of 4 runs, or else contiguous slices ((2, 8192, 2048): 22.9 us in
+    // slices, 25.9 us in 32 chunks).
+    int chunk_runs = tunables().fwd_cl_chunk_runs;
+    if (chunk_runs == 0) {
+        chunk_runs = 8;
+        if ((int64_t)blocks < (int64_t)8 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = 4;
+        if ((int64_t)blocks < (int64_t)8 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = -1;
+    }
+    g.blocks_per_chunk = chunk_runs <= 0 ? 0u : (uint32_t)(chunk_runs / 4 > 0 ? chunk_runs / 4 : 1) * g.waves_per_row;
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
+    if (g.blocks_per_chunk != 0)
+        g.blocks_per_xcd = (g.blocks_per_xcd + g.blocks_per_chunk - 1) / g.blocks_per_chunk * g.blocks_per_chunk;
+    if ((int64_t)g.blocks_per_xcd * kXcds * kBlock >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
     VarlenTail tail = {};
     tail.first_block = g.blocks_per_xcd * kXcds;
     if (gather != nullptr) {

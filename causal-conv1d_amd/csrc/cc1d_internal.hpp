@@ -55,6 +55,7 @@ inline bool varlen_fits_fwd_launch(const cc1d_fwd_params &f, const cc1d_varlen_p
 struct Tunables {
     int32_t fwd_cl_rows = 0;
     int32_t fwd_cl_half_vec = 0;
+    int32_t fwd_cl_chunk_runs = 0;
     int32_t bwd_cl_rows = 0;
     int32_t fwd_cf_vecs = 0;
     int32_t bwd_cf_parts = 0;
