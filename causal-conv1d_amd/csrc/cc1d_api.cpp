@@ -101,6 +101,7 @@ int cc1d_set_tunable(const char *name, int32_t value) {
     else if (!std::strcmp(name, "fwd_cl_half_vec")) t.fwd_cl_half_vec = value;
     else if (!std::strcmp(name, "fwd_cl_chunk_runs")) t.fwd_cl_chunk_runs = value;
     else if (!std::strcmp(name, "bwd_cl_rows")) t.bwd_cl_rows = value;
+    else if (!std::strcmp(name, "bwd_cl_chunk_runs")) t.bwd_cl_chunk_runs = value;
     else if (!std::strcmp(name, "fwd_cf_vecs")) t.fwd_cf_vecs = value;
     else if (!std::strcmp(name, "bwd_cf_parts")) t.bwd_cf_parts = value;
     else return CC1D_ERR_UNKNOWN_TUNABLE;
@@ -114,6 +115,7 @@ int cc1d_get_tunable(const char *name, int32_t *value) {
     else if (!std::strcmp(name, "fwd_cl_half_vec")) *value = t.fwd_cl_half_vec;
     else if (!std::strcmp(name, "fwd_cl_chunk_runs")) *value = t.fwd_cl_chunk_runs;
     else if (!std::strcmp(name, "bwd_cl_rows")) *value = t.bwd_cl_rows;
+    else if (!std::strcmp(name, "bwd_cl_chunk_runs")) *value = t.bwd_cl_chunk_runs;
     else if (!std::strcmp(name, "fwd_cf_vecs")) *value = t.fwd_cf_vecs;
     else if (!std::strcmp(name, "bwd_cf_parts")) *value = t.bwd_cf_parts;
     else return CC1D_ERR_UNKNOWN_TUNABLE;

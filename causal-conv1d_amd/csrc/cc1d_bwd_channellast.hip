@@ -52,6 +52,7 @@ struct BwdClGeom {
     uint32_t waves_per_row;   // ceil(n_colgroups / 64): workgroups side by side on one row
     uint32_t total;           // batch * n_quads * waves_per_row workgroups
     uint32_t blocks_per_xcd;  // grid size / 8
+    uint32_t blocks_per_chunk; // workgroups an XCD takes in a row before the next XCD's (0: its whole slice)
     int32_t w_mode;           // weights_mode: 0 general loader, 1 / 2 packed taps
 };
 
@@ -371,8 +372,12 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
     // Partial sums of wavefronts 1..3, one float per lane and term.
     __shared__ float partial[kRunsPerBlock - 1][(W + 1) * CH][kWave];
 
-    // XCD x executes workgroups x, x+8, x+16, ...; give it the x-th contiguous slice.
-    const uint32_t block = (blockIdx.x % kXcds) * g.blocks_per_xcd + blockIdx.x / kXcds;
+    // XCD x executes workgroups x, x+8, x+16, ...; give it chunks of consecutive runs, the 8 XCDs
+    // side by side on 8 neighbouring chunks (or, blocks_per_chunk == 0, the x-th contiguous slice).
+    const uint32_t xcd = blockIdx.x % kXcds, nth = blockIdx.x / kXcds;
+    const uint32_t block = g.blocks_per_chunk == 0
+                               ? xcd * g.blocks_per_xcd + nth
+                               : ((nth / g.blocks_per_chunk) * kXcds + xcd) * g.blocks_per_chunk + nth % g.blocks_per_chunk;
     // A workgroup takes 64 adjacent vector-columns of four consecutive runs of one sequence,
     // one run per wavefront: a wavefront's row range and the sub-sequence ids it reads are
     // scalars.  Neighbouring workgroups take neighbouring columns of the same rows.
@@ -526,6 +531,19 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     if (total * kBlock >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
     g.total = (uint32_t)total;
     g.blocks_per_xcd = (uint32_t)((total + kXcds - 1) / kXcds);
+    // Workgroup order, as in the forward: chunks of 8 runs (two workgroup rows), of 4 where the
+    // launch has fewer than eight such chunks per XCD, else one contiguous slice per XCD.
+    int chunk_runs = tunables().bwd_cl_chunk_runs;
+    if (chunk_runs == 0) {
+        chunk_runs = 8;
+        if (total < (int64_t)8 * kXcds * (chunk_runs / kRunsPerBlock) * g.waves_per_row) chunk_runs = 4;
+        if (total < (int64_t)8 * kXcds * (chunk_runs / kRunsPerBlock) * g.waves_per_row) chunk_runs = -1;
+    }
+    g.blocks_per_chunk = chunk_runs <= 0 ? 0u
+                                         : (uint32_t)(chunk_runs / kRunsPerBlock > 0 ? chunk_runs / kRunsPerBlock : 1) * g.waves_per_row;
+    if (g.blocks_per_chunk != 0)
+        g.blocks_per_xcd = (g.blocks_per_xcd + g.blocks_per_chunk - 1) / g.blocks_per_chunk * g.blocks_per_chunk;
+    if ((int64_t)g.blocks_per_xcd * kXcds * kBlock >= ((int64_t)1 << 31)) return false;
     g.w_mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     return true;
 }

@@ -57,6 +57,7 @@ struct Tunables {
     int32_t fwd_cl_half_vec = 0;
     int32_t fwd_cl_chunk_runs = 0;
     int32_t bwd_cl_rows = 0;
+    int32_t bwd_cl_chunk_runs = 0;
     int32_t fwd_cf_vecs = 0;
     int32_t bwd_cf_parts = 0;
 };
