@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the causal conv1d hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu] [--no-rotated]
 
 Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill shape
 (bf16, batch 8, dim 5376, seqlen 2048, channel-last, width 4, bias, SiLU, seq_idx with
@@ -323,6 +323,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
+    ap.add_argument("--no-rotated", action="store_true", help="skip the headline over rotating buffer sets")
     ap.add_argument("--rows", type=int, default=0, help="override rows per lane run (sweeps)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of x (a kernel of known size, to scale profiler counters)")
@@ -392,7 +393,7 @@ def main():
         for ln in open(traffic_file):
             if ln.startswith("traffic_bytes_per_launch:"):
                 line["roofline"]["traffic"] = int(float(ln.split(":")[1]))
-    if not args.no_others:
+    if not args.no_others and not args.no_rotated:
         # The same call over six rotating sets of x and out (2.1 GB): every launch then meets cold
         # address translations and caches, as the layers of a model do; next to it PyTorch's
         # elementwise add over the same sets (the same bytes in, the same bytes out).

@@ -531,12 +531,14 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     if (total * kBlock >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
     g.total = (uint32_t)total;
     g.blocks_per_xcd = (uint32_t)((total + kXcds - 1) / kXcds);
-    // Workgroup order, as in the forward: chunks of 8 runs (two workgroup rows), of 4 where the
-    // launch has fewer than eight such chunks per XCD, else one contiguous slice per XCD.
+    // Workgroup order, as in the forward: chunks of 4 runs (one workgroup row; 8 runs measured 1-2 %
+    // behind), or one contiguous slice per XCD where the launch has fewer than eight chunks per XCD.
+    // Slices -> chunks: (8, 5376, 2048) bf16 91.5 -> 90.0 us, (4, 4096, 4096) 77.0 -> 72.6 us,
+    // (16, 2048, 2048) 79.0 -> 73.4 us, (8, 10240, 2048) 177.8 -> 173.4 us.
     int chunk_runs = tunables().bwd_cl_chunk_runs;
+    if (chunk_runs == 0 && p.x_dtype == CC1D_F32) chunk_runs = -1;   // measured on 16-bit tensors only
     if (chunk_runs == 0) {
-        chunk_runs = 8;
-        if (total < (int64_t)8 * kXcds * (chunk_runs / kRunsPerBlock) * g.waves_per_row) chunk_runs = 4;
+        chunk_runs = 4;
         if (total < (int64_t)8 * kXcds * (chunk_runs / kRunsPerBlock) * g.waves_per_row) chunk_runs = -1;
     }
     g.blocks_per_chunk = chunk_runs <= 0 ? 0u

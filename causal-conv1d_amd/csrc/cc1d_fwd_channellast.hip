@@ -460,12 +460,22 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     // chunks per XCD take chunks of 4 runs, or else contiguous slices ((2, 8192, 2048): 22.9 us in
     // slices, 25.9 us in 32 chunks).
     int chunk_runs = tunables().fwd_cl_chunk_runs;
-    if (chunk_runs == 0) {
+    // Rows wider than 32 wavefronts gain nothing from chunks, and the headline shape (42 wavefronts
+    // a row, one batch entry per XCD) measured 55.3-55.5 us in slices against 56.7-57.0 us in chunks.
+    if (chunk_runs == 0 && g.waves_per_row > 32) chunk_runs = -1;
+    if (chunk_runs == 0 && p.x_dtype == CC1D_F32) {
+        // fp32 rows (twice the bytes, fewer wavefronts per CU) measured best in chunks of 16 runs, from
+        // four chunks per XCD on: (4, 2048, 4096) 42.5 us in slices, 46.6 in chunks of 8, 41.8 in chunks of
+        // 16 (cold 48.1 / 55.5 / 48.3); (16, 2048, 2048) 79.6 / 81.5 / 78.0 us (cold 98 / 102 / 92.6).
+        chunk_runs = 16;
+        if ((int64_t)blocks < (int64_t)4 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = -1;
+    } else if (chunk_runs == 0) {
         chunk_runs = 8;
         if ((int64_t)blocks < (int64_t)8 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = 4;
         if ((int64_t)blocks < (int64_t)8 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = -1;
     }
     g.blocks_per_chunk = chunk_runs <= 0 ? 0u : (uint32_t)(chunk_runs / 4 > 0 ? chunk_runs / 4 : 1) * g.waves_per_row;
+    if (chunk_runs < -1) g.blocks_per_chunk = (uint32_t)(-chunk_runs);   // sweeps: chunks of so many workgroups
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     if (g.blocks_per_chunk != 0)
         g.blocks_per_xcd = (g.blocks_per_xcd + g.blocks_per_chunk - 1) / g.blocks_per_chunk * g.blocks_per_chunk;

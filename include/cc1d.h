@@ -236,7 +236,8 @@ int cc1d_abi_version(void);
  *   "fwd_cl_half_vec" -1 = the channel-last forward reads its taps with the general loader even
  *                   when they are packed
  *   "fwd_cl_chunk_runs" consecutive runs an XCD takes before the next XCD's in the channel-last
- *                   forward's workgroup order (a multiple of 4; -1 = one contiguous slice per XCD)
+ *                   forward's workgroup order (a multiple of 4; -1 = one contiguous slice per XCD;
+ *                   -n, n > 1 = chunks of n workgroups)
  *   "bwd_cl_rows"   same for the channel-last backward
  *   "bwd_cl_chunk_runs" as "fwd_cl_chunk_runs", for the channel-last backward
  *   "fwd_cf_vecs"   16-byte vectors per wave segment in the channel-first forward
