@@ -536,10 +536,14 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     // Slices -> chunks: (8, 5376, 2048) bf16 91.5 -> 90.0 us, (4, 4096, 4096) 77.0 -> 72.6 us,
     // (16, 2048, 2048) 79.0 -> 73.4 us, (8, 10240, 2048) 177.8 -> 173.4 us.
     int chunk_runs = tunables().bwd_cl_chunk_runs;
-    if (chunk_runs == 0 && p.x_dtype == CC1D_F32) chunk_runs = -1;   // measured on 16-bit tensors only
+    // fp32 rows of at most 16 wavefronts measured best in chunks of 16 runs, from four chunks per XCD
+    // on: (4, 2048, 4096) 79.1 us in slices, 75.1 in chunks of 4, 70.5 in chunks of 16; (16, 2048, 2048)
+    // 148.2 / 138.9 / 133.7 us; wider fp32 rows in chunks of 4 ((8, 5376, 2048) 174.1 -> 173.0 us).
     if (chunk_runs == 0) {
         chunk_runs = 4;
-        if (total < (int64_t)8 * kXcds * (chunk_runs / kRunsPerBlock) * g.waves_per_row) chunk_runs = -1;
+        if (p.x_dtype == CC1D_F32 && g.waves_per_row <= 16 &&
+            total >= (int64_t)4 * kXcds * (16 / kRunsPerBlock) * g.waves_per_row) chunk_runs = 16;
+        if (chunk_runs == 4 && total < (int64_t)8 * kXcds * g.waves_per_row) chunk_runs = -1;
     }
     g.blocks_per_chunk = chunk_runs <= 0 ? 0u
                                          : (uint32_t)(chunk_runs / kRunsPerBlock > 0 ? chunk_runs / kRunsPerBlock : 1) * g.waves_per_row;
