@@ -197,6 +197,28 @@ def test_bwd_is_bit_reproducible(pkg, gpu_device, channel_last):
     check(first, ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bwd_workgroup_order_does_not_change_results(pkg, gpu_device, cc1d_lib, dtype):
+    """Channel-last backward: slices or chunks of runs per XCD, same bits in every gradient (the
+    partial sums of dweight keep their places in the second stage's order)."""
+    lib = cabi.declare(cc1d_lib)
+    g = gen(13)
+    x = make_x(3, 1160, 1237, dtype, True, g)
+    dout = make_x(3, 1160, 1237, dtype, True, g, sliced=False)
+    w, b = make_wb(1160, 4, True, g)
+    outs = []
+    try:
+        for chunk in (-1, 0, 4, 8, 16, 64):
+            assert lib.cc1d_set_tunable(b"bwd_cl_chunk_runs", chunk) == 0
+            outs.append([t.cpu() for t in run_gpu(pkg, gpu_device, x, w, b, dout, act="silu")[:3]])
+    finally:
+        lib.cc1d_set_tunable(b"bwd_cl_chunk_runs", 0)
+    for o in outs[1:]:
+        for a, r in zip(o, outs[0]):
+            assert torch.equal(a, r)
+    check(tuple(outs[0]) + (None,), orc.bwd(x, w, b, dout, activation="silu"), dtype)
+
+
 @pytest.mark.parametrize("channel_last", [False, True])
 def test_bwd_c_abi_accumulates_into_dweight(gpu_device, cc1d_lib, channel_last):
     """Through the C ABI with a caller-owned workspace: dweight / dbias are added to, as the

@@ -263,6 +263,30 @@ def test_fwd_launch_geometry_does_not_change_results(pkg, gpu_device, cc1d_lib, 
     assert torch.equal(outs[0][2], fin)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fwd_workgroup_order_does_not_change_results(pkg, gpu_device, cc1d_lib, dtype):
+    """The channel-last forward hands its workgroups to the XCDs in contiguous slices or in chunks
+    of runs, by shape; every order covers every run exactly once: same bits, ragged last run and
+    a launch that is no whole number of chunks included."""
+    lib = cabi.declare(cc1d_lib)
+    g = gen(12)
+    x = make_x(3, 1160, 1237, dtype, True, g).to(gpu_device)
+    w, b = (t.to(gpu_device) for t in make_wb(1160, 4, True, g))
+    seq = random_seq_idx(3, 1237, g, pad=True).to(gpu_device)
+    outs = []
+    try:
+        for chunk in (-1, 0, 4, 8, 16, 64, -3, -7):
+            assert lib.cc1d_set_tunable(b"fwd_cl_chunk_runs", chunk) == 0
+            o = pkg.causal_conv1d_fn(x, w, b, seq_idx=seq, activation="silu")
+            _, f = pkg.causal_conv1d_fn(x, w, b, return_final_states=True, activation="silu")
+            outs.append((o.cpu(), f.cpu()))
+    finally:
+        lib.cc1d_set_tunable(b"fwd_cl_chunk_runs", 0)
+    for o in outs[1:]:
+        assert torch.equal(o[0], outs[0][0]) and torch.equal(o[1], outs[0][1])
+    assert_close(outs[0][0], orc.fwd_seq_idx(x.cpu(), w.cpu(), b.cpu(), seq.cpu(), activation="silu"), dtype, "out")
+
+
 def test_fwd_through_the_c_abi_on_a_side_stream(gpu_device, cc1d_lib):
     """The C ABI alone: raw pointers, element strides and an explicit stream handle."""
     lib = cabi.declare(cc1d_lib)
