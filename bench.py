@@ -2,6 +2,7 @@
 """Benchmark of the causal conv1d hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu] [--no-rotated]
+                    [--no-sustained] [--only update]
 
 Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill shape
 (bf16, batch 8, dim 5376, seqlen 2048, channel-last, width 4, bias, SiLU, seq_idx with
@@ -11,7 +12,12 @@ Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill 
                      algorithmic bytes count every input element read once and every
                      output element written once (x, out, seq_idx, weight, bias)
   roofline ......... the same bytes over the average kernel time measured with HIP events
-                     around the timed launches, against the 8 TB/s HBM3E peak
+                     around the timed launches, against the 8 TB/s HBM3E peak.  `frac` is the
+                     warm burst the K timed steps are (one set of buffers, a few milliseconds of
+                     load); `frac_sustained` the same call over 400 back-to-back launches, past
+                     the point where the clock settles; `frac_rotated` over six rotating sets of
+                     x and out (2.1 GB), where every launch meets cold caches and address
+                     translations, as the layers of a model do
   cpu_baseline ..... the PyTorch oracle (F.conv1d per packed sub-sequence) timed on this
                      host's cores on the same inputs
   others ........... µs per call and GB/s of the remaining shapes: decode-step update
@@ -132,6 +138,38 @@ def config_c5b(width, dtype, channel_last, batch=4, dim=2048, seqlen=4096):
     return dict(x=make_x(batch, dim, seqlen, dtype, channel_last, 50 + width), weight=w, bias=b)
 
 
+def kernel_sources_sha16(names):
+    """First 16 hex digits of the SHA-256 over the named kernel sources, in order."""
+    import hashlib
+    h = hashlib.sha256()
+    for n in names:
+        with open(os.path.join(PKG_DIR, "csrc", n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profile_figures(profile, sources):
+    """`key: number` lines of a committed rocprofv3 summary under profiles/, or {} when the
+    summary is missing or was made from other kernel sources than the ones in the tree (it
+    names them by hash): a counter figure is only reported next to the code it was read on."""
+    path = os.path.join(ROOT, "profiles", profile)
+    if not os.path.exists(path):
+        return {}
+    figs = {}
+    for ln in open(path):
+        key, sep, val = ln.partition(":")
+        if sep and key.strip().replace("_", "").isalnum() and " " not in key.strip():
+            figs[key.strip()] = val.strip()
+    if figs.get("kernel_sources_sha16") != kernel_sources_sha16(sources):
+        return {}
+    figs["profile"] = "profiles/" + profile
+    return figs
+
+
+FWD_CL_SOURCES = ("cc1d_fwd_channellast.hip", "cc1d_device.hpp", "cc1d_varlen_gather.hpp")
+UPDATE_SOURCES = ("cc1d_update.hip", "cc1d_device.hpp")
+
+
 def nbytes(*tensors):
     return sum(t.numel() * t.element_size() for t in tensors if t is not None)
 
@@ -173,12 +211,22 @@ def clone_sets(cfg, bytes_per_set, max_sets=64):
     return [{k: cp(v) for k, v in cfg.items()} for _ in range(n)]
 
 
+def update_algorithmic_bytes(cfg, circular):
+    """Decode step: x, out, taps and bias once; the state's W-1 window rows read and, linear, every
+    state row written (S = W-1 here), or, circular, one row written plus cache_seqlens."""
+    x, st = cfg["x"], cfg["conv_state"]
+    n = nbytes(x, x, cfg["weight"], cfg["bias"])
+    if circular:
+        return n + 3 * nbytes(x) + nbytes(x) + nbytes(cfg["cache_seqlens"])
+    return n + 2 * nbytes(st)
+
+
 def gbs(n_bytes, us):
     return n_bytes / us * 1e-3 if us > 0 else 0.0
 
 
 # ---------------------------------------------------------------------- the other shapes
-def bench_others(ext, dev, steps, warmup):
+def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False):
     import torch
     res = {}
 
@@ -190,31 +238,37 @@ def bench_others(ext, dev, steps, warmup):
             res[name].update(extra)
 
     # C3: decode-step update, linear and circular.
+    prof = profile_figures("update_step_decode_device_time.txt", UPDATE_SOURCES)
     for circular in (False, True):
         name = "update_circular_s8" if circular else "update_linear_s3"
         cfg = to_dev(config_c3(circular), dev)
         x, st = cfg["x"], cfg["conv_state"]
-        n_bytes = nbytes(x, x, cfg["weight"], cfg["bias"])
-        if circular:
-            n_bytes += 3 * nbytes(x) + nbytes(x) + nbytes(cfg["cache_seqlens"])   # window read + 1 row written
-        else:
-            n_bytes += 2 * nbytes(st)
+        n_bytes = update_algorithmic_bytes(cfg, circular)
         out = torch.empty_like(x)
         cs = cfg.get("cache_seqlens")
         us, wall = time_gpu(lambda i: ext.causal_conv1d_update(x, st, cfg["weight"], cfg["bias"], out, True, cs, None),
                             steps, warmup)
-        sets = clone_sets(cfg, nbytes(x, st, x))
-        outs = [torch.empty_like(s["x"]) for s in sets]
-        def rot(i):
-            s = sets[i % len(sets)]
-            ext.causal_conv1d_update(s["x"], s["conv_state"], s["weight"], s["bias"], outs[i % len(sets)], True,
-                                     s.get("cache_seqlens"), None)
-        us_rot, _ = time_gpu(rot, steps, warmup)
-        record(name, us, n_bytes, {"us_rotated": round(us_rot, 3),
-                                   "GBps_rotated": round(gbs(n_bytes, us_rot), 1),
-                                   "frac_of_hbm_peak_rotated": round(gbs(n_bytes, us_rot) / HBM_PEAK_GBS, 4),
-                                   "rotated_sets": len(sets), "us_wall_per_call": round(wall, 2)})
-        del sets, outs
+        extra = {"us_wall_per_call": round(wall, 2)}
+        if rotated:
+            sets = clone_sets(cfg, nbytes(x, st, x))
+            outs = [torch.empty_like(s["x"]) for s in sets]
+            def rot(i):
+                s = sets[i % len(sets)]
+                ext.causal_conv1d_update(s["x"], s["conv_state"], s["weight"], s["bias"], outs[i % len(sets)], True,
+                                         s.get("cache_seqlens"), None)
+            us_rot, _ = time_gpu(rot, steps, warmup)
+            extra.update({"us_rotated": round(us_rot, 3), "GBps_rotated": round(gbs(n_bytes, us_rot), 1),
+                          "frac_of_hbm_peak_rotated": round(gbs(n_bytes, us_rot) / HBM_PEAK_GBS, 4),
+                          "rotated_sets": len(sets)})
+            del sets, outs
+        # Device duration of the warm launches by rocprofv3 (no dispatch gap in it), from the
+        # committed summary of `bench.py --only update`, while the kernel is the one profiled.
+        key = "circular_us_device_avg" if circular else "linear_us_device_avg"
+        if key in prof:
+            extra.update({"us_device_rocprof": float(prof[key]), "us_device_rocprof_source": prof["profile"]})
+        record(name, us, n_bytes, extra)
+    if only_update:
+        return res
 
     # What this box charges for any launch of the decode step's size, measured the same way:
     # a device-to-device copy moving as many bytes as the linear step (half read, half written)
@@ -263,7 +317,7 @@ def bench_others(ext, dev, steps, warmup):
     states = torch.empty(64, 3, 5376, device=dev, dtype=torch.bfloat16).transpose(1, 2)
     n_bytes = 2 * nbytes(states) + nbytes(cfg["cu_seqlens"])
     us, _ = time_gpu(lambda i: ext.causal_conv1d_varlen_states(cfg["x"], cfg["cu_seqlens"], states, 3), steps, warmup)
-    record("varlen_states_c5a", us, n_bytes)
+    record("varlen_states_c5a", us, n_bytes, {"bound": "launch: 4 MB move in well under the ~2.5 us a dispatch costs"})
     del cfg
 
     # C5b: forward sweep over width x dtype x layout.
@@ -324,7 +378,10 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-rotated", action="store_true", help="skip the headline over rotating buffer sets")
-    ap.add_argument("--rows", type=int, default=0, help="override rows per lane run (sweeps)")
+    ap.add_argument("--no-sustained", action="store_true", help="skip the 400-launch sustained figure")
+    ap.add_argument("--only", choices=["update"], default=None,
+                    help="time nothing but the warm decode-step launches (linear, then circular): the "
+                         "command whose rocprofv3 kernel trace gives their device durations")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of x (a kernel of known size, to scale profiler counters)")
     args = ap.parse_args()
@@ -337,16 +394,16 @@ def main():
         sys.exit("bench.py: no GPU visible; the benchmark has no CPU fallback")
     import causal_conv1d_cuda as ext          # fails loudly if the extension was not built
     dev = torch.device("cuda:0")
+    if args.only == "update":
+        res = bench_others(ext, dev, args.steps, args.warmup, rotated=False, only_update=True)
+        print(json.dumps({"only": "update", "steps": args.steps, "warmup": args.warmup, "others": res}), flush=True)
+        return
 
     cfg_cpu = config_c2()
     cfg = to_dev(cfg_cpu, dev)
     x, w, b, seq = cfg["x"], cfg["weight"], cfg["bias"], cfg["seq_idx"]
     out = torch.empty_like(x)
     n_bytes = nbytes(x, out, seq, w, b)
-    if args.rows:
-        import ctypes
-        lib = ctypes.CDLL(os.path.join(PKG_DIR, "libcc1d.so"))
-        lib.cc1d_set_tunable(b"fwd_cl_rows", ctypes.c_int32(args.rows))
 
     def step(i):
         ext.causal_conv1d_fwd(x, w, b, seq, None, out, None, True)
@@ -388,11 +445,21 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbs(n_bytes, us), 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs(n_bytes, us) / HBM_PEAK_GBS, 4), "traffic": None},
     }
-    traffic_file = os.path.join(ROOT, "profiles", "fwd_channellast_prefill_traffic.txt")
-    if os.path.exists(traffic_file):
-        for ln in open(traffic_file):
-            if ln.startswith("traffic_bytes_per_launch:"):
-                line["roofline"]["traffic"] = int(float(ln.split(":")[1]))
+    # HBM bytes per launch by FETCH_SIZE / WRITE_SIZE: only rocprofv3 can read those, so the figure
+    # comes from the committed summary, and only while the kernel sources are the ones it was
+    # read on (the summary names them by hash); otherwise null.
+    prof = profile_figures("fwd_channellast_prefill_traffic.txt", FWD_CL_SOURCES)
+    if "traffic_bytes_per_launch" in prof:
+        line["roofline"]["traffic"] = int(float(prof["traffic_bytes_per_launch"]))
+        line["roofline"]["traffic_source"] = {"profile": prof["profile"],
+                                              "kernel_sources_sha16": prof["kernel_sources_sha16"]}
+    if not args.no_sustained:
+        # The same call 400 times back to back (about 25 ms of load): the clock settles after the
+        # first few milliseconds, which the K timed steps above mostly end before.
+        sus_us, _ = time_gpu(step, 400, 0)
+        line["config"]["us_per_call_sustained"] = round(sus_us, 3)
+        line["config"]["sustained_steps"] = 400
+        line["roofline"]["frac_sustained"] = round(gbs(n_bytes, sus_us) / HBM_PEAK_GBS, 4)
     if not args.no_others and not args.no_rotated:
         # The same call over six rotating sets of x and out (2.1 GB): every launch then meets cold
         # address translations and caches, as the layers of a model do; next to it PyTorch's
@@ -404,6 +471,7 @@ def main():
         line["config"].update({"us_per_call_rotated": round(rot_us, 3), "rotated_sets": 6,
                                "GBps_rotated": round(gbs(n_bytes, rot_us), 1),
                                "us_torch_add_rotated": round(add_us, 3)})
+        line["roofline"]["frac_rotated"] = round(gbs(n_bytes, rot_us) / HBM_PEAK_GBS, 4)
         del sets
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg_cpu, n_bytes, gpu_out_host)

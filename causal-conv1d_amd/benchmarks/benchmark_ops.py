@@ -10,11 +10,20 @@ backward here is always a fixed-order two-stage sum.
   python benchmark_ops.py --op update --batch 256 --dim 5376 --state-len 8 --circular
   python benchmark_ops.py --op varlen --batch 64 --dim 5376 --seqlen 1024
   python benchmark_ops.py --op prefill --batch 16 --dim 5376 --seqlen 256
+
+With --rocprof DIR the same measurement runs once more as a child process under
+`rocprofv3 --kernel-trace --stats -d DIR -o benchmark_ops -- python3 benchmark_ops.py ...` and the
+device-side duration of every kernel of this library in that run (average, median, minimum,
+maximum over its dispatches, without the gaps between dispatches that event timing includes) is
+printed below the table; the raw trace stays in DIR.
 """
 import argparse
 import gc
+import glob
 import os
+import sqlite3
 import statistics
+import subprocess
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
@@ -57,6 +66,52 @@ def peak_mb(fn):
     return (torch.cuda.max_memory_allocated() - base) / 2**20
 
 
+def kernel_durations(trace_dir):
+    """{kernel name: [durations in us]} of this library's kernels from the rocprofv3 result
+    database(s) under trace_dir (the `kernels` view: name, start and end in nanoseconds)."""
+    per_kernel = {}
+    for db_path in sorted(glob.glob(os.path.join(trace_dir, "**", "*_results.db"), recursive=True)):
+        db = sqlite3.connect(db_path)
+        try:
+            rows = db.execute("select name, start, end from kernels order by start").fetchall()
+        finally:
+            db.close()
+        for name, start, end in rows:
+            if "cc1d" in name:
+                short = name.replace("void cc1d::(anonymous namespace)::", "").replace("cc1d::", "")
+                short = short[:short.find("(")] if "(" in short else short
+                per_kernel.setdefault(short, []).append((end - start) * 1e-3)
+    return per_kernel
+
+
+def run_under_rocprof(trace_dir, argv):
+    """The same command line, minus --rocprof, as a child of rocprofv3; returns the lines of the
+    kernel table.  Called before anything here has touched the GPU."""
+    child_args, skip = [], False
+    for arg in argv:
+        if skip:
+            skip = False
+        elif arg == "--rocprof":
+            skip = True
+        elif not arg.startswith("--rocprof="):
+            child_args.append(arg)
+    os.makedirs(trace_dir, exist_ok=True)
+    cmd = ["rocprofv3", "--kernel-trace", "--stats", "-d", trace_dir, "-o", "benchmark_ops", "--",
+           "python3", os.path.abspath(__file__)] + child_args
+    print("+ " + " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        sys.exit("rocprofv3 run failed (%d):\n%s" % (res.returncode, res.stdout[-4000:]))
+    per_kernel = kernel_durations(trace_dir)
+    if not per_kernel:
+        sys.exit("rocprofv3 run left no kernel records of this library under " + trace_dir)
+    lines = ["device-side kernel durations (rocprofv3 --kernel-trace), microseconds",
+             "%6s %9s %9s %9s %9s  %s" % ("calls", "avg", "median", "min", "max", "kernel")]
+    for name, d in sorted(per_kernel.items(), key=lambda kv: -sum(kv[1])):
+        lines.append("%6d %9.2f %9.2f %9.2f %9.2f  %s" % (len(d), sum(d) / len(d), statistics.median(d), min(d), max(d), name))
+    return lines
+
+
 def nbytes(*ts):
     return sum(t.numel() * t.element_size() for t in ts if t is not None)
 
@@ -81,7 +136,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--rep", type=int, default=50)
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--rocprof", metavar="DIR", default=None,
+                    help="also run under rocprofv3 --kernel-trace into DIR and print device-side kernel durations")
     a = ap.parse_args()
+    # The profiled run goes first, while this process has not touched the GPU yet.
+    profile_lines = run_under_rocprof(a.rocprof, sys.argv[1:]) if a.rocprof else []
 
     dev = "cuda"
     dtype = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[a.dtype]
@@ -153,7 +212,9 @@ def main():
     print("op=%s batch=%d dim=%d seqlen=%d width=%d dtype=%s channel_last=%s seq_idx=%s states=%s bias=%s act=%s"
           % (a.op, B, D, L, W, a.dtype, a.channel_last, a.seq_idx, a.states, not a.no_bias, a.activation))
     print("%10s %12s %10s %12s %10s" % ("us/call", "bytes moved", "GB/s", "% of 8 TB/s", "peak MB"))
-    print("%10.2f %12d %10.1f %12.1f %10.1f" % (us, moved, gbs, 100 * gbs / HBM_PEAK_GBS, mb))
+    print("%10.2f %12d %10.1f %12.1f %10.1f" % (us, moved, gbs, 100 * gbs / HBM_PEAK_GBS, mb), flush=True)
+    if profile_lines:
+        print("\n".join(profile_lines), flush=True)
 
 
 if __name__ == "__main__":

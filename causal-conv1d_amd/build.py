@@ -85,7 +85,13 @@ def build_kernels(force=False, extra_flags=(), lib_path=None):
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         list(ex.map(_run, jobs))
     if force or jobs or not _newer(lib_path, objs):
-        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path] + objs)
+        # Linked by the host compiler, not by hipcc: hipcc's link step writes the toolkit's own
+        # lib directory into RUNPATH, and a process that has PyTorch loaded must bind to the HIP
+        # runtime PyTorch ships (same soname, libamdhip64.so.7), never map a second one.  With
+        # no RUNPATH the NEEDED entry resolves to the runtime already in the process, or to the
+        # system's (ld.so.conf) when there is none.
+        _run([os.environ.get("CXX", "g++"), "-shared", "-fPIC", "-o", lib_path] + objs +
+             ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-ldl"])
     return lib_path
 
 

@@ -3,6 +3,8 @@
 // reference's host binding (csrc/causal_conv1d.cpp:158-199, 273-327, 475-542); layout
 // selection follows csrc/causal_conv1d.cpp:176,296.  Nothing here allocates or
 // synchronises; validation never touches the GPU, so it can run on a GPU-less host.
+#include <dlfcn.h>
+
 #include <cstring>
 
 #include "cc1d.h"
@@ -55,6 +57,127 @@ int check_common(const P *p) {
     return CC1D_OK;
 }
 
+// Byte range [lo, hi) a (batch, dim, width-1) states tensor with non-negative strides covers.
+void states_extent(const void *base, int64_t sb, int64_t sc, int64_t sl, const cc1d_fwd_params &p,
+                   uintptr_t *lo, uintptr_t *hi) {
+    auto span = [](int64_t n, int64_t stride) { return n > 1 ? (uint64_t)(n - 1) * (uint64_t)(stride < 0 ? -stride : stride) : 0u; };
+    const uint64_t last = span(p.batch, sb) + span(p.dim, sc) + span(p.width - 1, sl);
+    *lo = reinterpret_cast<uintptr_t>(base);
+    *hi = *lo + (uintptr_t)((last + 1) * (uint64_t)elem_bytes(p.x_dtype));
+}
+
+// Do initial_states and final_states share an element?  Disjoint byte ranges: no.  Otherwise, for two
+// views with the same strides (two slices of one buffer), exactly: they share an element iff the
+// distance between their bases is db*sb + dc*sc + dl*sl for index differences inside the shape.
+// Views with different strides whose byte ranges intersect count as overlapping.
+bool states_overlap(const cc1d_fwd_params &p) {
+    uintptr_t a0, a1, b0, b1;
+    states_extent(p.initial_states, p.init_stride_b, p.init_stride_c, p.init_stride_l, p, &a0, &a1);
+    states_extent(p.final_states, p.final_stride_b, p.final_stride_c, p.final_stride_l, p, &b0, &b1);
+    if (!(a0 < b1 && b0 < a1)) return false;
+    const int64_t sb = p.init_stride_b, sc = p.init_stride_c, sl = p.init_stride_l;
+    const bool same_strides = (p.batch <= 1 || sb == p.final_stride_b) && (p.dim <= 1 || sc == p.final_stride_c) &&
+                              (p.width <= 2 || sl == p.final_stride_l);
+    const int64_t eb = elem_bytes(p.x_dtype);
+    const int64_t bytes = (int64_t)b0 - (int64_t)a0;
+    if (!same_strides || bytes % eb != 0) return true;
+    const int64_t delta = bytes / eb;
+    for (int64_t dl = -(p.width - 2); dl <= p.width - 2; ++dl) {
+        for (int64_t db = -((int64_t)p.batch - 1); db <= (int64_t)p.batch - 1; ++db) {
+            const int64_t rest = delta - (p.width > 2 ? dl * sl : 0) - (p.batch > 1 ? db * sb : 0);
+            if (p.dim <= 1 || sc == 0) {
+                if (rest == 0) return true;
+            } else if (rest % sc == 0 && rest / sc > -(int64_t)p.dim && rest / sc < (int64_t)p.dim) {
+                return true;
+            }
+        }
+    }
+    return false;
+}
+
+// ---- batch slicing ---------------------------------------------------------------------------
+// A launcher refuses, before launching anything, a problem that needs more work items than one
+// grid holds (CC1D_ERR_TOO_LARGE).  Every batch entry is independent, so the front then halves
+// the batch until the pieces fit and launches them one after the other on the same stream: the
+// reference's grid(batch, dim) launch has no such ceiling, and neither has this library.
+const void *advance(const void *base, int64_t elems, int bytes_per_elem) {
+    return base == nullptr ? nullptr : static_cast<const char *>(base) + elems * bytes_per_elem;
+}
+void *advance(void *base, int64_t elems, int bytes_per_elem) {
+    return base == nullptr ? nullptr : static_cast<char *>(base) + elems * bytes_per_elem;
+}
+
+cc1d_fwd_params batch_slice(const cc1d_fwd_params &p, int b0, int n) {
+    cc1d_fwd_params q = p;
+    const int eb = elem_bytes(p.x_dtype);
+    q.batch = n;
+    q.x = advance(p.x, b0 * p.x_stride_b, eb);
+    q.out = advance(p.out, b0 * p.out_stride_b, eb);
+    q.seq_idx = static_cast<const int32_t *>(advance(p.seq_idx, (int64_t)b0 * p.seqlen, 4));
+    q.initial_states = advance(p.initial_states, b0 * p.init_stride_b, eb);
+    q.final_states = advance(p.final_states, b0 * p.final_stride_b, eb);
+    return q;
+}
+
+cc1d_bwd_params batch_slice(const cc1d_bwd_params &p, int b0, int n) {
+    cc1d_bwd_params q = p;
+    const int eb = elem_bytes(p.x_dtype);
+    q.batch = n;
+    q.x = advance(p.x, b0 * p.x_stride_b, eb);
+    q.dout = advance(p.dout, b0 * p.dout_stride_b, eb);
+    q.dx = advance(p.dx, b0 * p.dx_stride_b, eb);
+    q.seq_idx = static_cast<const int32_t *>(advance(p.seq_idx, (int64_t)b0 * p.seqlen, 4));
+    q.initial_states = advance(p.initial_states, b0 * p.init_stride_b, eb);
+    q.dfinal_states = advance(p.dfinal_states, b0 * p.dfinal_stride_b, eb);
+    q.dinitial_states = advance(p.dinitial_states, b0 * p.dinit_stride_b, eb);
+    if (b0 > 0) q.overwrite_dweight = 0;              // later slices add to what the first one stored
+    return q;
+}
+
+cc1d_update_params batch_slice(const cc1d_update_params &p, int b0, int n) {
+    cc1d_update_params q = p;
+    const int eb = elem_bytes(p.x_dtype);
+    q.batch = n;
+    q.x = advance(p.x, b0 * p.x_stride_b, eb);
+    q.out = advance(p.out, b0 * p.out_stride_b, eb);
+    q.cache_seqlens = static_cast<const int32_t *>(advance(p.cache_seqlens, b0, 4));
+    if (p.conv_state_indices != nullptr) {
+        q.conv_state_indices = static_cast<const int32_t *>(advance(p.conv_state_indices, b0, 4));
+    } else {
+        q.conv_state = advance(p.conv_state, b0 * p.state_stride_b, eb);
+        q.state_batch = n;
+    }
+    return q;
+}
+
+// launch(params) for the whole batch, or for halves of it (recursively) while it answers
+// CC1D_ERR_TOO_LARGE.  Slices run in batch order.
+template <typename P, typename F>
+int launch_in_batch_slices(const P &p, F &&launch) {
+    const int st = launch(p);
+    if (st != CC1D_ERR_TOO_LARGE || p.batch < 2) return st;
+    const int head = p.batch / 2;
+    const int first = launch_in_batch_slices(batch_slice(p, 0, head), launch);
+    if (first != CC1D_OK) return first;
+    return launch_in_batch_slices(batch_slice(p, head, p.batch - head), launch);
+}
+
+size_t bwd_workspace_one_launch(const cc1d_bwd_params &p) {
+    return is_channel_last(p.x_stride_c, p.x_stride_l) ? bwd_channellast_workspace_bytes(p)
+                                                       : bwd_channelfirst_workspace_bytes(p);
+}
+bool bwd_fits_one_launch(const cc1d_bwd_params &p) {
+    return is_channel_last(p.x_stride_c, p.x_stride_l) ? bwd_channellast_fits(p) : bwd_channelfirst_fits(p);
+}
+// The workspace the largest slice needs: slices run one after the other and share it.
+size_t bwd_workspace_sliced(const cc1d_bwd_params &p) {
+    if (bwd_fits_one_launch(p) || p.batch < 2) return bwd_workspace_one_launch(p);
+    const int head = p.batch / 2;
+    const size_t a = bwd_workspace_sliced(batch_slice(p, 0, head));
+    const size_t b = bwd_workspace_sliced(batch_slice(p, head, p.batch - head));
+    return a > b ? a : b;
+}
+
 template <typename P>
 bool is_empty(const P *p) {
     return p->batch == 0 || p->dim == 0 || p->seqlen == 0;
@@ -94,31 +217,50 @@ const char *cc1d_strerror(int status) {
     }
 }
 
+int cc1d_hip_runtime_path(char *path, size_t size) {
+    if (path == nullptr || size == 0) return CC1D_ERR_NULL_POINTER;
+    path[0] = '\0';
+    Dl_info info;
+    if (dladdr(reinterpret_cast<const void *>(&hipLaunchKernel), &info) == 0 || info.dli_fname == nullptr)
+        return CC1D_ERR_LAUNCH;
+    const size_t n = std::strlen(info.dli_fname);
+    if (n + 1 > size) return CC1D_ERR_SHAPE;
+    std::memcpy(path, info.dli_fname, n + 1);
+    return CC1D_OK;
+}
+
+namespace {
+Knob *find_knob(const char *name) {
+    Tunables &t = tunables();
+    static const struct { const char *name; Knob Tunables::*knob; } table[] = {
+        {"fwd_cl_rows", &Tunables::fwd_cl_rows},
+        {"fwd_cl_half_vec", &Tunables::fwd_cl_half_vec},
+        {"fwd_cl_chunk_runs", &Tunables::fwd_cl_chunk_runs},
+        {"bwd_cl_rows", &Tunables::bwd_cl_rows},
+        {"bwd_cl_chunk_runs", &Tunables::bwd_cl_chunk_runs},
+        {"fwd_cf_vecs", &Tunables::fwd_cf_vecs},
+        {"bwd_cf_parts", &Tunables::bwd_cf_parts},
+        {"launch_limit_shift", &Tunables::launch_limit_shift},
+    };
+    for (const auto &e : table)
+        if (!std::strcmp(name, e.name)) return &(t.*(e.knob));
+    return nullptr;
+}
+}  // namespace
+
 int cc1d_set_tunable(const char *name, int32_t value) {
     if (name == nullptr) return CC1D_ERR_NULL_POINTER;
-    Tunables &t = tunables();
-    if (!std::strcmp(name, "fwd_cl_rows")) t.fwd_cl_rows = value;
-    else if (!std::strcmp(name, "fwd_cl_half_vec")) t.fwd_cl_half_vec = value;
-    else if (!std::strcmp(name, "fwd_cl_chunk_runs")) t.fwd_cl_chunk_runs = value;
-    else if (!std::strcmp(name, "bwd_cl_rows")) t.bwd_cl_rows = value;
-    else if (!std::strcmp(name, "bwd_cl_chunk_runs")) t.bwd_cl_chunk_runs = value;
-    else if (!std::strcmp(name, "fwd_cf_vecs")) t.fwd_cf_vecs = value;
-    else if (!std::strcmp(name, "bwd_cf_parts")) t.bwd_cf_parts = value;
-    else return CC1D_ERR_UNKNOWN_TUNABLE;
+    Knob *k = find_knob(name);
+    if (k == nullptr) return CC1D_ERR_UNKNOWN_TUNABLE;
+    k->set(value);
     return CC1D_OK;
 }
 
 int cc1d_get_tunable(const char *name, int32_t *value) {
     if (name == nullptr || value == nullptr) return CC1D_ERR_NULL_POINTER;
-    const Tunables &t = tunables();
-    if (!std::strcmp(name, "fwd_cl_rows")) *value = t.fwd_cl_rows;
-    else if (!std::strcmp(name, "fwd_cl_half_vec")) *value = t.fwd_cl_half_vec;
-    else if (!std::strcmp(name, "fwd_cl_chunk_runs")) *value = t.fwd_cl_chunk_runs;
-    else if (!std::strcmp(name, "bwd_cl_rows")) *value = t.bwd_cl_rows;
-    else if (!std::strcmp(name, "bwd_cl_chunk_runs")) *value = t.bwd_cl_chunk_runs;
-    else if (!std::strcmp(name, "fwd_cf_vecs")) *value = t.fwd_cf_vecs;
-    else if (!std::strcmp(name, "bwd_cf_parts")) *value = t.bwd_cf_parts;
-    else return CC1D_ERR_UNKNOWN_TUNABLE;
+    const Knob *k = find_knob(name);
+    if (k == nullptr) return CC1D_ERR_UNKNOWN_TUNABLE;
+    *value = *k;
     return CC1D_OK;
 }
 
@@ -135,6 +277,16 @@ int cc1d_validate_fwd(const cc1d_fwd_params *p) {
                            p->out_stride_c, p->out_stride_l);
     if (st != CC1D_OK) return st;
     if (p->seq_idx != nullptr && !cl) return CC1D_ERR_SEQ_IDX_LAYOUT;
+    // initial_states and final_states may be one and the same tensor (csrc/causal_conv1d.h:44 of the
+    // reference: a chunked prefill that keeps a single state buffer): same address, same strides.
+    // Every kernel reads a row's initial_states and writes its final_states from one wavefront, reads
+    // first.  Two different views that share memory have no such guarantee and are refused.
+    if (p->initial_states != nullptr && p->final_states != nullptr && p->width > 1) {
+        const bool same = p->initial_states == p->final_states && p->init_stride_b == p->final_stride_b &&
+                          p->init_stride_c == p->final_stride_c &&
+                          (p->width == 2 || p->init_stride_l == p->final_stride_l);
+        if (!same && states_overlap(*p)) return CC1D_ERR_STATE_LAYOUT;
+    }
     return CC1D_OK;
 }
 
@@ -143,8 +295,10 @@ int cc1d_fwd(const cc1d_fwd_params *p, cc1d_stream_t stream) {
     if (st != CC1D_OK) return st;
     if (is_empty(p)) return CC1D_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return is_channel_last(p->x_stride_c, p->x_stride_l) ? launch_fwd_channellast(*p, nullptr, s)
-                                                         : launch_fwd_channelfirst(*p, s);
+    return launch_in_batch_slices(*p, [s](const cc1d_fwd_params &q) {
+        return is_channel_last(q.x_stride_c, q.x_stride_l) ? launch_fwd_channellast(q, nullptr, s)
+                                                           : launch_fwd_channelfirst(q, s);
+    });
 }
 
 int cc1d_fwd_varlen_states(const cc1d_fwd_params *fwd, const cc1d_varlen_params *gather, cc1d_stream_t stream) {
@@ -160,8 +314,10 @@ int cc1d_fwd_varlen_states(const cc1d_fwd_params *fwd, const cc1d_varlen_params 
     hipStream_t s = static_cast<hipStream_t>(stream);
     // One launch when the forward is channel-last and the gather moves whole 16-byte vectors
     // of elements as wide as the forward's; two launches otherwise.
-    if (is_channel_last(fwd->x_stride_c, fwd->x_stride_l) && varlen_fits_fwd_launch(*fwd, *gather))
-        return launch_fwd_channellast(*fwd, gather, s);
+    if (is_channel_last(fwd->x_stride_c, fwd->x_stride_l) && varlen_fits_fwd_launch(*fwd, *gather)) {
+        st = launch_fwd_channellast(*fwd, gather, s);
+        if (st != CC1D_ERR_TOO_LARGE) return st;      // too large for one grid: two calls, the forward in slices
+    }
     st = cc1d_fwd(fwd, stream);
     return st != CC1D_OK ? st : launch_varlen_states(*gather, s);
 }
@@ -198,8 +354,7 @@ int cc1d_bwd_workspace_bytes(const cc1d_bwd_params *p, size_t *bytes) {
     const int st = cc1d_validate_bwd(p);
     if (st != CC1D_OK) return st;
     if (is_empty(p)) return CC1D_OK;
-    *bytes = is_channel_last(p->x_stride_c, p->x_stride_l) ? bwd_channellast_workspace_bytes(*p)
-                                                            : bwd_channelfirst_workspace_bytes(*p);
+    *bytes = bwd_workspace_sliced(*p);
     return CC1D_OK;
 }
 
@@ -216,8 +371,10 @@ int cc1d_bwd(const cc1d_bwd_params *p, void *workspace, size_t workspace_bytes, 
     if (need > 0 && (workspace == nullptr || !aligned16(workspace) || workspace_bytes < need))
         return CC1D_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return is_channel_last(p->x_stride_c, p->x_stride_l) ? launch_bwd_channellast(*p, workspace, s)
-                                                         : launch_bwd_channelfirst(*p, workspace, s);
+    return launch_in_batch_slices(*p, [s, workspace](const cc1d_bwd_params &q) {
+        return is_channel_last(q.x_stride_c, q.x_stride_l) ? launch_bwd_channellast(q, workspace, s)
+                                                           : launch_bwd_channelfirst(q, workspace, s);
+    });
 }
 
 // -------------------------------------------------------------------------- update
@@ -237,7 +394,8 @@ int cc1d_update(const cc1d_update_params *p, cc1d_stream_t stream) {
     const int st = cc1d_validate_update(p);
     if (st != CC1D_OK) return st;
     if (is_empty(p)) return CC1D_OK;
-    return launch_update(*p, static_cast<hipStream_t>(stream));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return launch_in_batch_slices(*p, [s](const cc1d_update_params &q) { return launch_update(q, s); });
 }
 
 // ------------------------------------------------------------------- varlen states

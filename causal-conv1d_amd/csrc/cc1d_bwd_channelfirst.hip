@@ -868,8 +868,8 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + vec - 1) / vec;
     const int64_t max_steps = (max_vecs + kWave - 1) / kWave;     // 64-vector steps per row
     // About 16 waves on each of 256 CUs when the problem allows it.
-    int64_t parts = tunables().bwd_cf_parts > 0 ? tunables().bwd_cf_parts
-                                                : (4096 + p.dim - 1) / p.dim;
+    const int32_t forced_parts = tunables().bwd_cf_parts;
+    int64_t parts = forced_parts > 0 ? forced_parts : (4096 + p.dim - 1) / p.dim;
     const int64_t max_parts = (int64_t)p.batch * max_steps;
     if (parts > max_parts) parts = max_parts;
     if (parts < 1) parts = 1;
@@ -902,7 +902,7 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
     // instead, down to eight steps of work per wavefront: (32, 1536, 2048) bf16 126 -> 107 us,
     // (64, 768, 1024) 69 -> 65 us, (8, 5376, 2048) fp32 205 -> 175 us, (1, 5376, 131072) bf16 875 -> 690 us;
     // other wave counts measured best as they are.
-    if (tunables().bwd_cf_parts <= 0 && p.dim * parts > 4096 && 2 * p.dim * parts < 3 * 4096) {
+    if (forced_parts <= 0 && p.dim * parts > 4096 && 2 * p.dim * parts < 3 * 4096) {
         int64_t finer = p.batch * max_steps / 8;
         if (finer > 64) finer = 64;
         if (finer > parts) parts = finer;
@@ -925,7 +925,7 @@ BwdCfGeom make_geom(const cc1d_bwd_params &p) {
 template <int DT>
 int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStream_t stream) {
     const int64_t waves = (int64_t)p.dim * g.n_parts;
-    if (waves >= ((int64_t)1 << 25)) return CC1D_ERR_TOO_LARGE;
+    if (waves >= wave_limit()) return CC1D_ERR_TOO_LARGE;
     const uint32_t blocks = (uint32_t)((waves + (kBlock / kWave) - 1) / (kBlock / kWave));
     if (g.streaming == 3) {                           // short rows, several batch entries to a wavefront
         switch (p.width) {
@@ -973,6 +973,10 @@ size_t bwd_channelfirst_workspace_bytes(const cc1d_bwd_params &p) {
     const BwdCfGeom g = make_geom(p);
     if (g.n_parts == 1) return 0;
     return (size_t)g.n_parts * (p.width + 1) * (size_t)p.dim * sizeof(float);
+}
+
+bool bwd_channelfirst_fits(const cc1d_bwd_params &p) {
+    return (int64_t)p.dim * make_geom(p).n_parts < wave_limit();
 }
 
 int launch_bwd_channelfirst(const cc1d_bwd_params &p, void *workspace, hipStream_t stream) {

@@ -528,7 +528,7 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
     g.n_quads = (g.n_runs + kRunsPerBlock - 1) / kRunsPerBlock;
     g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
     const int64_t total = (int64_t)p.batch * g.n_quads * g.waves_per_row;    // workgroups
-    if (total * kBlock >= ((int64_t)1 << 31) - kXcds * kBlock) return false;
+    if (total * kBlock >= thread_limit() - kXcds * kBlock) return false;
     g.total = (uint32_t)total;
     g.blocks_per_xcd = (uint32_t)((total + kXcds - 1) / kXcds);
     // Workgroup order, as in the forward: chunks of 4 runs (one workgroup row; 8 runs measured 1-2 %
@@ -549,7 +549,7 @@ bool make_geom(const cc1d_bwd_params &p, BwdClGeom &g) {
                                          : (uint32_t)(chunk_runs / kRunsPerBlock > 0 ? chunk_runs / kRunsPerBlock : 1) * g.waves_per_row;
     if (g.blocks_per_chunk != 0)
         g.blocks_per_xcd = (g.blocks_per_xcd + g.blocks_per_chunk - 1) / g.blocks_per_chunk * g.blocks_per_chunk;
-    if ((int64_t)g.blocks_per_xcd * kXcds * kBlock >= ((int64_t)1 << 31)) return false;
+    if ((int64_t)g.blocks_per_xcd * kXcds * kBlock >= thread_limit()) return false;
     g.w_mode = weights_mode(p.weight, p.bias, p.w_dtype, p.x_dtype, p.w_stride_c, p.w_stride_w, p.width);
     return true;
 }
@@ -590,6 +590,11 @@ size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p) {
     BwdClGeom g;
     if (!make_geom(p, g)) return 0;
     return (size_t)p.batch * g.n_quads * (p.width + 1) * (size_t)p.dim * sizeof(float);
+}
+
+bool bwd_channellast_fits(const cc1d_bwd_params &p) {
+    BwdClGeom g;
+    return make_geom(p, g);
 }
 
 int launch_bwd_channellast(const cc1d_bwd_params &p, void *workspace, hipStream_t stream) {

@@ -402,6 +402,15 @@ __device__ __forceinline__ float from_next_lane(float v, float lane63_fill) {
 __device__ __forceinline__ float read_lane(float v, int lane) {
     return bitcast<float>(__builtin_amdgcn_readlane(bitcast<int>(v), lane));
 }
+// Every vector-memory load this wavefront has issued so far has returned.  Used in front of the
+// final_states stores of the forward kernels: final_states may be the very buffer initial_states
+// were read from (a chunked prefill that keeps one state tensor), the wavefront that reads a
+// row's initial_states is the one that writes its final_states, and with this wait the reads are
+// complete before the first such store is issued.
+__device__ __forceinline__ void wait_for_loads() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Sum over the 64 lanes of a wave in a fixed butterfly order (deterministic).
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -474,7 +474,7 @@ int launch_short(const cc1d_fwd_params &p, int n_vecs, bool aligned, hipStream_t
     while ((1 << lanes_log2) < n_vecs) ++lanes_log2;
     const int64_t rows = (int64_t)p.batch * p.dim;
     const int64_t threads = rows << lanes_log2;
-    if (threads >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+    if (threads >= thread_limit()) return CC1D_ERR_TOO_LARGE;
     const dim3 grid((uint32_t)((threads + kBlock - 1) / kBlock)), block(kBlock);
     const uint32_t n_rows = (uint32_t)rows;
 #define CC1D_SHORT2(WIDTH, SILU_ON)                                                                                  \
@@ -697,12 +697,17 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     // Rows that are not whole vectors on one grid take the same lanes with element accesses:
     // (16, 5376, 100) bf16 45.9 -> 25.4 us, (64, 2048, 60) 63.7 -> 16.4 us, (256, 5376, 4) 360 -> 11.9 us.
     const int64_t short_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
-    if (short_vecs <= 64 && tunables().fwd_cf_vecs <= 0) {
+    const int32_t forced_vecs = tunables().fwd_cf_vecs;
+    if (short_vecs <= 64 && forced_vecs <= 0) {
         const bool aligned = same_grid && on_grid && p.seqlen % vec == 0;
         // A contiguous tensor of rows that are not whole vectors, but at least one: whole vectors of
         // the flat array, (16, 5376, 100) bf16 25.4 -> 13.5 us, (16, 5376, 130) 28.5 -> 16.2 us, (64, 2048, 60) 16.4 -> 11.6 us.
         const int64_t n_elems = rows * p.seqlen;
-        const bool flat = !aligned && p.seqlen >= vec && n_elems < ((int64_t)1 << 31) &&
+        // (Not when final_states may be the buffer initial_states come from: in the flat walk the
+        // lane that reads a row's initial_states and the lane that writes its final_states can sit in
+        // different wavefronts.)
+        const bool states_in_and_out = p.initial_states != nullptr && p.final_states != nullptr;
+        const bool flat = !aligned && !states_in_and_out && p.seqlen >= vec && n_elems < ((int64_t)1 << 31) &&
                           aligned16(p.x) && aligned16(p.out) &&
                           (p.dim == 1 || (p.x_stride_c == p.seqlen && p.out_stride_c == p.seqlen)) &&
                           (p.batch == 1 || (p.x_stride_b == (int64_t)p.dim * p.seqlen &&
@@ -721,8 +726,8 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
         }
     }
     int64_t vps;
-    if (tunables().fwd_cf_vecs > 0) {
-        vps = tunables().fwd_cf_vecs;
+    if (forced_vecs > 0) {
+        vps = forced_vecs;
     } else {
         // Enough waves to cover 256 CUs about 16 deep; otherwise one wave per row, except that
         // long rows (1024 vectors and up) are cut into segments of 256 vectors: many short-lived
@@ -741,7 +746,7 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     g.vecs_per_seg = (int32_t)vps;
     g.n_segs = (int32_t)((max_vecs + vps - 1) / vps);
     const int64_t total = rows * g.n_segs;
-    if (total >= ((int64_t)1 << 25)) return CC1D_ERR_TOO_LARGE;   // total*64 threads must fit 2^31
+    if (total >= wave_limit()) return CC1D_ERR_TOO_LARGE;   // total*64 threads must fit 2^31
     g.total_waves = (uint32_t)total;
     switch (p.x_dtype) {
         case CC1D_F32: return launch_dtype<CC1D_F32>(p, g, stream);

@@ -344,9 +344,12 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         }
     }
 
-    // final_states[b, c, i] = xpad[L-(W-1)+i]: the last run re-reads those few rows
-    // (just streamed, still in cache) instead of tracking them through the loop.
-    if (p.final_states != nullptr && run == g.n_runs - 1) {
+    // final_states[b, c, i] = xpad[L-(W-1)+i], copied from x (or initial_states where L < W-1)
+    // by the wavefront of the FIRST run, the one that read initial_states as its halo: the two
+    // may be one buffer, and inside one wavefront the reads are complete before the stores.
+    if (p.final_states != nullptr && run == 0) {
+        wait_for_loads();
+        raw_t fin[W - 1];
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) {
             const int t = L - (W - 1) + i;
@@ -357,9 +360,13 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
                 r = load_state_row<DT, CH>(p.initial_states, p.init_stride_b, p.init_stride_c,
                                            p.init_stride_l, b, c0, t + (W - 1));
             }
-            store_state_row<DT, CH>(p.final_states, p.final_stride_b, p.final_stride_c,
-                                    p.final_stride_l, b, c0, i, r);
+            fin[i] = r;
         }
+        wait_for_loads();                             // rows shorter than W-1 re-read initial_states above
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i)
+            store_state_row<DT, CH>(p.final_states, p.final_stride_b, p.final_stride_c,
+                                    p.final_stride_l, b, c0, i, fin[i]);
     }
 }
 
@@ -447,7 +454,7 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     if (g.rows_per_run == 0) return CC1D_ERR_TOO_LARGE;
     g.n_runs = (p.seqlen + g.rows_per_run - 1) / g.rows_per_run;
     const int64_t total = (int64_t)p.batch * g.n_runs * g.waves_per_row;
-    if (total * kWave >= ((int64_t)1 << 31) - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
+    if (total * kWave >= thread_limit() - kXcds * kBlock) return CC1D_ERR_TOO_LARGE;
     g.total = (uint32_t)total;
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     // Workgroup order: an XCD takes chunks of `chunk_runs` consecutive runs (all their column
@@ -479,14 +486,14 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     if (g.blocks_per_chunk != 0)
         g.blocks_per_xcd = (g.blocks_per_xcd + g.blocks_per_chunk - 1) / g.blocks_per_chunk * g.blocks_per_chunk;
-    if ((int64_t)g.blocks_per_xcd * kXcds * kBlock >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+    if ((int64_t)g.blocks_per_xcd * kXcds * kBlock >= thread_limit()) return CC1D_ERR_TOO_LARGE;
     VarlenTail tail = {};
     tail.first_block = g.blocks_per_xcd * kXcds;
     if (gather != nullptr) {
         tail.p = *gather;
         tail.n_colgroups = (uint32_t)(gather->dim / vec_elems(gather->x_dtype));
         const int64_t threads = (int64_t)gather->batch * gather->state_len * tail.n_colgroups;
-        if (threads + (int64_t)tail.first_block * kBlock >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+        if (threads + (int64_t)tail.first_block * kBlock >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         tail.total = (uint32_t)threads;
     }
     switch (p.x_dtype) {

@@ -8,6 +8,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "cc1d.h"
 
 namespace cc1d {
@@ -52,16 +54,30 @@ inline bool varlen_fits_fwd_launch(const cc1d_fwd_params &f, const cc1d_varlen_p
     return varlen_vec_ok(v) && elem_bytes(v.x_dtype) == elem_bytes(f.x_dtype);
 }
 
+// Launch-heuristic overrides for sweeps and for the tests that prove results do not depend on
+// launch geometry.  0 = the built-in choice.  Each knob is an independent relaxed atomic: a
+// launch reads it once, a concurrent cc1d_set_tunable from another thread is a data-race-free
+// store, and no knob changes what a launch computes, only how it is cut into workgroups.
+struct Knob {
+    std::atomic<int32_t> v{0};
+    operator int32_t() const { return v.load(std::memory_order_relaxed); }
+    void set(int32_t x) { v.store(x, std::memory_order_relaxed); }
+};
 struct Tunables {
-    int32_t fwd_cl_rows = 0;
-    int32_t fwd_cl_half_vec = 0;
-    int32_t fwd_cl_chunk_runs = 0;
-    int32_t bwd_cl_rows = 0;
-    int32_t bwd_cl_chunk_runs = 0;
-    int32_t fwd_cf_vecs = 0;
-    int32_t bwd_cf_parts = 0;
+    Knob fwd_cl_rows, fwd_cl_half_vec, fwd_cl_chunk_runs, bwd_cl_rows, bwd_cl_chunk_runs, fwd_cf_vecs,
+        bwd_cf_parts, launch_limit_shift;
 };
 Tunables &tunables();
+
+// The kernels number their work items with 32 bits, so one launch holds fewer than 2^31 threads
+// (2^25 wavefronts).  A launcher whose problem needs more returns CC1D_ERR_TOO_LARGE before it
+// launches anything, and the C-ABI front then cuts the batch into slices that fit.  The knob
+// lowers the limit (by that many bits) so that tests reach the slicing with small tensors.
+inline int64_t thread_limit() {
+    const int32_t shift = tunables().launch_limit_shift;
+    return ((int64_t)1 << 31) >> (shift > 0 && shift <= 24 ? shift : 0);
+}
+inline int64_t wave_limit() { return thread_limit() / 64; }
 
 inline int launch_status() {
     return hipGetLastError() == hipSuccess ? CC1D_OK : CC1D_ERR_LAUNCH;
@@ -72,6 +88,9 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream);
 
 size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p);
 size_t bwd_channelfirst_workspace_bytes(const cc1d_bwd_params &p);
+// false: the launcher would answer CC1D_ERR_TOO_LARGE (and launch nothing).
+bool bwd_channellast_fits(const cc1d_bwd_params &p);
+bool bwd_channelfirst_fits(const cc1d_bwd_params &p);
 int launch_bwd_channellast(const cc1d_bwd_params &p, void *ws, hipStream_t stream);
 int launch_bwd_channelfirst(const cc1d_bwd_params &p, void *ws, hipStream_t stream);
 // Second stage of both backward layouts: ordered sum of the workspace planes into dweight/dbias.

@@ -630,14 +630,14 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
     if (vec) {
         const uint32_t ncg = (uint32_t)(p.dim / Elem<DT>::kVec);
         const int64_t total = (int64_t)p.batch * ncg;
-        if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+        if (total >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
         const int w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
         if (circ) hipLaunchKernelGGL((update_vec_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, p, ncg, (uint32_t)total, w_fast);
         else hipLaunchKernelGGL((update_vec_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, p, ncg, (uint32_t)total, w_fast);
     } else {
         const int64_t total = (int64_t)p.batch * p.dim;
-        if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
+        if (total >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
         if (circ) hipLaunchKernelGGL((update_generic_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, p, (uint32_t)total);
         else hipLaunchKernelGGL((update_generic_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, p, (uint32_t)total);

@@ -56,7 +56,7 @@ typedef enum cc1d_status {
     CC1D_ERR_WORKSPACE = -13,        /* workspace NULL, misaligned or too small */
     CC1D_ERR_BIAS_MISMATCH = -14,    /* bias given without dbias or the reverse (causal_conv1d.cpp:281) */
     CC1D_ERR_SEQ_IDX_STATES = -15,   /* seq_idx combined with initial/final states */
-    CC1D_ERR_TOO_LARGE = -16,        /* a launch dimension exceeds what the grid can express */
+    CC1D_ERR_TOO_LARGE = -16,        /* one batch entry alone exceeds what a grid can express */
     CC1D_ERR_LAUNCH = -17,           /* the HIP runtime refused the launch */
     CC1D_ERR_UNKNOWN_TUNABLE = -18
 } cc1d_status;
@@ -230,8 +230,19 @@ int cc1d_fwd_varlen_states(const cc1d_fwd_params *fwd, const cc1d_varlen_params 
 const char *cc1d_strerror(int status);
 int cc1d_abi_version(void);
 
-/* Benchmarking hooks: override a launch heuristic (0 restores the built-in choice).
- * Process-global, not thread-safe, meant for sweeps only.  Known names:
+/* Diagnostic, host-only: writes the file name of the HIP runtime library this library's launches
+ * go through (the shared object that defines hipLaunchKernel for it) into path[0..size), always
+ * NUL-terminated.  A process must hold exactly one HIP runtime: a host that also uses PyTorch
+ * loads PyTorch (or PyTorch's own libamdhip64.so) BEFORE this library, so that this library's
+ * NEEDED entry binds to that copy, and can check here that it did.  No counterpart in the
+ * reference, whose kernels are linked into the PyTorch extension itself.  Returns CC1D_OK,
+ * CC1D_ERR_NULL_POINTER, or CC1D_ERR_SHAPE when the name does not fit. */
+int cc1d_hip_runtime_path(char *path, size_t size);
+
+/* Benchmarking and test hooks: override a launch heuristic (0 restores the built-in choice).
+ * Process-global; each knob is an atomic integer read once per launch, so setting one while
+ * another thread launches is safe, and no knob changes what a launch computes (only how the
+ * work is cut into workgroups and launches).  Known names:
  *   "fwd_cl_rows"   rows of seqlen walked by one lane of the channel-last forward
  *   "fwd_cl_half_vec" -1 = the channel-last forward reads its taps with the general loader even
  *                   when they are packed
@@ -242,6 +253,12 @@ int cc1d_abi_version(void);
  *   "bwd_cl_chunk_runs" as "fwd_cl_chunk_runs", for the channel-last backward
  *   "fwd_cf_vecs"   16-byte vectors per wave segment in the channel-first forward
  *   "bwd_cf_parts"  partitions of (batch x seqlen) per channel in the channel-first backward
+ *   "launch_limit_shift" n: one launch holds at most 2^(31-n) threads instead of 2^31 (n <= 24), so
+ *                   that small tensors exercise the batch slicing below
+ *
+ * A problem with more work items than one grid holds (2^31 threads) is cut along the batch into
+ * slices that fit, launched back to back on the stream; forward, backward and update accept any
+ * batch.  CC1D_ERR_TOO_LARGE is left for a single batch entry that does not fit one launch.
  */
 int cc1d_set_tunable(const char *name, int32_t value);
 int cc1d_get_tunable(const char *name, int32_t *value);

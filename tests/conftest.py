@@ -1,11 +1,15 @@
 """Shared test plumbing: path set-up, the `gpu` marker, and loading of the in-tree native
 libraries (built on demand when nothing has been built yet)."""
 import ctypes
+import faulthandler
 import glob
 import os
 import sys
 
 import pytest
+
+# A crash on the host (segmentation fault, abort) must leave its Python stack in the log.
+faulthandler.enable(all_threads=True)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PKG_DIR = os.path.join(ROOT, "causal-conv1d_amd")

@@ -30,7 +30,7 @@ def test_every_declared_symbol_is_exported(lib):
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"\b(cc1d_[a-z_0-9]+)\s*\(", text)
-    assert len(set(names)) == 14
+    assert len(set(names)) >= 15 and {'cc1d_fwd', 'cc1d_bwd', 'cc1d_update', 'cc1d_varlen_states'} <= set(names)
     for n in set(names):
         assert hasattr(lib, n), f"{n} declared in cc1d.h but not exported"
     assert lib.cc1d_abi_version() == 1
@@ -101,6 +101,39 @@ def test_validate_fwd_paths(lib):
     assert v(p) == OK
     p, _k = _fwd(); p.batch = 0; p.x = None
     assert v(p) == OK and lib.cc1d_fwd(p, None) == OK      # empty problem: nothing to launch
+
+
+def test_validate_fwd_states_that_share_memory(lib):
+    """initial_states and final_states may be one tensor (same address, same strides); two
+    different views are accepted when they share no element and refused when they do."""
+    v = lib.cc1d_validate_fwd
+    B, D, W = 2, 16, 4
+
+    def with_states(init, fin):
+        p, keep = _fwd(B=B, D=D, W=W, channel_last=True)
+        cabi._set3(p, "init", "initial_states", init)
+        cabi._set3(p, "final", "final_states", fin)
+        return p, (keep, init, fin)
+
+    state = torch.zeros(B, W - 1, D).transpose(1, 2)
+    p, _k = with_states(state, state)
+    assert v(p) == OK                                   # one buffer
+    p, _k = with_states(state, torch.zeros(B, W - 1, D).transpose(1, 2))
+    assert v(p) == OK                                   # two allocations
+    big = torch.zeros(B, 8, D).transpose(1, 2)          # (B, D, 8): two windows of one cache
+    p, _k = with_states(big[:, :, 0:3], big[:, :, 3:6])
+    assert v(p) == OK                                   # interleaved in memory, no element in common
+    p, _k = with_states(big[:, :, 0:3], big[:, :, 2:5])
+    assert v(p) == E_STATE_LAYOUT                       # share position 2
+    p, _k = with_states(big[:, :, 2:5], big[:, :, 0:3])
+    assert v(p) == E_STATE_LAYOUT
+    p, _k = with_states(state, state.contiguous().transpose(1, 2)[:, :W - 1, :W - 1].new_zeros(B, D, W - 1))
+    assert v(p) == OK
+    flat = torch.zeros(B * D * (W - 1))
+    a = flat.as_strided((B, D, W - 1), (D * (W - 1), 1, D))          # dim fastest
+    c = flat.as_strided((B, D, W - 1), (D * (W - 1), W - 1, 1))      # seqlen fastest, same memory
+    p, _k = with_states(a, c)
+    assert v(p) == E_STATE_LAYOUT                       # same bytes under two different views
 
 
 def _bwd(channel_last=False, bias=True):

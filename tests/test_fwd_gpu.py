@@ -324,3 +324,51 @@ def test_fwd_error_behaviour(pkg, gpu_device):
                              return_final_states=True)
     empty = pkg.causal_conv1d_fn(torch.zeros(0, 16, 32, device=d), torch.zeros(16, 4, device=d))
     assert empty.shape == (0, 16, 32)
+
+
+@pytest.mark.parametrize("channel_last", [False, True], ids=["cf", "cl"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fwd_one_buffer_for_initial_and_final_states(pkg, gpu_device, dtype, channel_last):
+    """A chunked prefill that keeps ONE state tensor: initial_states and final_states_out are the
+    same buffer (allowed by the reference, csrc/causal_conv1d.h:44).  Chunks of many runs, of a few
+    rows, of fewer than width-1 rows and of odd lengths must reproduce the unchunked result bit
+    for bit, and leave the last width-1 inputs in the buffer."""
+    dev = gpu_device
+    g = gen(91)
+    B, D, W = 3, 264, 4
+    L = 1500 if channel_last else 1499
+    x = make_x(B, D, L, dtype, channel_last, g, sliced=False).to(dev)
+    w, b = (t.to(dev) for t in make_wb(D, W, True, g))
+    init = make_states(B, D, W - 1, dtype, g).to(dev)
+    whole, whole_fin = pkg.causal_conv1d_fn(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+    # chunks of 512, 8, 2, 1, 477 and about 500 positions; channel-first slices start off the
+    # 16-byte grid
+    cuts = [0, 512, 520, 522, 523, 1000, L]
+    for layout in ("dim_fastest", "len_fastest"):
+        state = (init.clone() if layout == "dim_fastest" else init.contiguous().clone())
+        outs = []
+        for lo, hi in zip(cuts[:-1], cuts[1:]):
+            o, fin = pkg.causal_conv1d_fn(x[:, :, lo:hi], w, b, initial_states=state, return_final_states=True,
+                                          final_states_out=state, activation="silu")
+            assert fin.data_ptr() == state.data_ptr()
+            outs.append(o)
+        assert torch.equal(torch.cat(outs, dim=2), whole), layout
+        assert torch.equal(state, whole_fin), layout
+    ref, ref_fin = orc.fwd(x.cpu(), w.cpu(), b.cpu(), initial_states=init.cpu(), return_final_states=True, activation="silu")
+    assert_close(whole, ref, dtype, "out")
+    assert torch.equal(whole_fin.cpu(), ref_fin)
+
+
+def test_fwd_on_a_side_stream_through_the_package(pkg, gpu_device):
+    """The binding launches on torch's current stream, whichever it is."""
+    dev = gpu_device
+    g = gen(92)
+    x = make_x(2, 128, 777, torch.bfloat16, True, g, sliced=False).to(dev)
+    w, b = (t.to(dev) for t in make_wb(128, 4, True, g))
+    ref = pkg.causal_conv1d_fn(x, w, b, activation="silu")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = pkg.causal_conv1d_fn(x, w, b, activation="silu")
+    side.synchronize()
+    assert torch.equal(got, ref)
