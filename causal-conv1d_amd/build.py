@@ -29,6 +29,7 @@ KERNEL_SOURCES = [
     "cc1d_fwd_channelfirst.hip",
     "cc1d_bwd_channellast.hip",
     "cc1d_bwd_channelfirst.hip",
+    "cc1d_bwd_noalloc.hip",
     "cc1d_update.hip",
     "cc1d_varlen_states.hip",
 ]

@@ -213,6 +213,7 @@ const char *cc1d_strerror(int status) {
         case CC1D_ERR_TOO_LARGE: return "problem too large for one launch";
         case CC1D_ERR_LAUNCH: return "HIP kernel launch failed";
         case CC1D_ERR_UNKNOWN_TUNABLE: return "unknown tunable name";
+        case CC1D_ERR_WORKSPACE_LIMIT: return "backward needs more workspace than the library's built-in array holds; use cc1d_bwd with a caller-owned workspace";
         default: return "unknown cc1d status";
     }
 }

@@ -58,7 +58,8 @@ typedef enum cc1d_status {
     CC1D_ERR_SEQ_IDX_STATES = -15,   /* seq_idx combined with initial/final states */
     CC1D_ERR_TOO_LARGE = -16,        /* one batch entry alone exceeds what a grid can express */
     CC1D_ERR_LAUNCH = -17,           /* the HIP runtime refused the launch */
-    CC1D_ERR_UNKNOWN_TUNABLE = -18
+    CC1D_ERR_UNKNOWN_TUNABLE = -18,
+    CC1D_ERR_WORKSPACE_LIMIT = -19   /* cc1d_bwd_noalloc: the problem needs more than the built-in workspace */
 } cc1d_status;
 
 /* Opaque stream handle: pass a hipStream_t (NULL = the default stream). */
@@ -152,6 +153,24 @@ int cc1d_validate_bwd(const cc1d_bwd_params *p);
 int cc1d_bwd_workspace_bytes(const cc1d_bwd_params *p, size_t *bytes);
 int cc1d_bwd(const cc1d_bwd_params *p, void *workspace, size_t workspace_bytes,
              cc1d_stream_t stream);
+
+/* The backward for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference, whose
+ * backward allocates its workspaces itself with at::zeros (csrc/causal_conv1d.cpp:396-429).
+ * Same kernels, same order of additions and same results as cc1d_bwd; the partial-sum workspace
+ * is a fixed array of CC1D_BWD_NOALLOC_MAX_WORKSPACE_BYTES inside this library's device image
+ * (one copy per GPU, held from the first use of the library on that GPU until the process ends).
+ * A problem whose cc1d_bwd_workspace_bytes() exceeds that size is refused with
+ * CC1D_ERR_WORKSPACE_LIMIT before anything is launched (16 MiB covers, for instance, the bf16
+ * prefill shape (8, 5376, 2048) channel-last at 13.8 MB; channel-first problems with dim >= 4096
+ * need none).  Calls no hipMalloc / hipFree and nothing that allocates.  The device that owns
+ * `stream` must be the current device.  All calls on one GPU share that GPU's array: calls that
+ * overlap in time on one GPU (different streams, no ordering between them) race; calls on one
+ * stream never do.  The array needs no clearing between calls (every plane that is read was
+ * written by the same call).  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress), so make it outside graph capture. */
+#define CC1D_BWD_NOALLOC_MAX_WORKSPACE_BYTES (16u * 1024u * 1024u)
+int cc1d_bwd_noalloc(const cc1d_bwd_params *p, cc1d_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * Decode-step update.  Replaces causal_conv1d_update (csrc/causal_conv1d.cpp:465-557)

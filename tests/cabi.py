@@ -151,6 +151,8 @@ def declare(lib):
     lib.cc1d_fwd.argtypes = [C.POINTER(FwdParams), vp]
     lib.cc1d_bwd_workspace_bytes.argtypes = [C.POINTER(BwdParams), C.POINTER(C.c_size_t)]
     lib.cc1d_bwd.argtypes = [C.POINTER(BwdParams), vp, C.c_size_t, vp]
+    if hasattr(lib, "cc1d_bwd_noalloc"):
+        lib.cc1d_bwd_noalloc.argtypes = [C.POINTER(BwdParams), vp]
     lib.cc1d_update.argtypes = [C.POINTER(UpdateParams), vp]
     lib.cc1d_varlen_states.argtypes = [C.POINTER(VarlenParams), vp]
     lib.cc1d_fwd_varlen_states.argtypes = [C.POINTER(FwdParams), C.POINTER(VarlenParams), vp]
