@@ -105,51 +105,26 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     const uint32_t rb = wave / g.waves_per_row;
     const int run = (int)(rb % (uint32_t)g.n_runs);
     const int b = (int)(rb / (uint32_t)g.n_runs);
-    const int c0 = (int)col * CH;
     const int L = p.seqlen;
     const int T = g.rows_per_run;                     // multiple of 2*U
     const int t0 = run * T;                           // < L by construction of n_runs
     const int last = L - 1 - t0;                      // last valid row of this run, run-relative
 
-    // With seq_idx the walk computes every row as if no sub-sequence boundary were near (no
-    // branch, no ids in the hot loop); the groups of U rows whose rows or window are not all of
-    // one non-negative id are redone with masked taps after the walk.  Which groups those are is
-    // found here, with all 64 lanes, a row per lane: lane i holds row i-(W-1) of a stretch of
-    // whole groups and flags it when its id differs from the row before or is negative (rows in
-    // front of the sequence count as id -1 when initial_states are given, as zeros, which no
-    // mask changes, otherwise); group k is redone when a flag falls into its rows or the W-2
-    // rows before them.  Where more than half of the groups are (sub-sequences of a few tokens),
-    // the walk is skipped and the masked pass takes the whole run.
-    uint32_t redo = 0;
-    bool dense = false;
-    if (HAS_SEQ) {
-        const int n_groups = T / U;
-        if (n_groups > 32) {
-            dense = true;
-        } else {
-            constexpr int kStretch = (kWave - (W - 1)) / U;            // groups per look
-            const int32_t *ids = seq_idx + (int64_t)b * L;
-            const int lane = threadIdx.x & (kWave - 1);
-            const bool init = p.initial_states != nullptr;
-            for (int k0 = 0; k0 < n_groups; k0 += kStretch) {
-                const int t_lane = t0 + k0 * U + lane - (W - 1);       // row of this lane
-                const int t = t_lane > L - 1 ? L - 1 : t_lane;
-                const int id = ids[t > 0 ? t : 0];
-                const int id_prev = ids[t > 1 ? t - 1 : 0];
-                const bool flag = t_lane > L - 1 ? false
-                                : t >= 0 ? (id < 0 || (t > 0 ? id != id_prev : init)) : init;
-                const uint64_t flags = __ballot(flag);
-                for (int k = 0; k < kStretch && k0 + k < n_groups; ++k)
-                    if ((flags >> (k * U + 1)) & ((1ull << (U + W - 2)) - 1)) redo |= 1u << (k0 + k);
-            }
-            int live = last / U + 1;                                   // groups with rows inside the sequence
-            live = live > n_groups ? n_groups : live;
-            redo &= live >= 32 ? ~0u : (1u << live) - 1u;
-            dense = 2 * __builtin_popcount(redo) > live;
-        }
-    }
-    if (col >= (uint32_t)g.n_colgroups) return;       // no cross-lane traffic below
+    // Lanes past the last column group (a row that is no whole number of wavefronts) shadow column
+    // group 0 until the wavefront's cross-lane work is done: every address they form is valid, and
+    // they leave before the first store.
+    const bool col_ok = col < (uint32_t)g.n_colgroups;
+    const int c0 = col_ok ? (int)col * CH : 0;
 
+    // With seq_idx, the ids of the run's first rows (a row per lane, see below) are the first thing
+    // requested: the look at them then waits for this one load, which finds its line in L2, and
+    // not for the halo rows behind it, which may come from HBM.
+    int first_ids = 0;
+    if (HAS_SEQ) {
+        const int t_lane = t0 + (int)(threadIdx.x & (kWave - 1)) - (W - 1);
+        const int t = t_lane > L - 1 ? L - 1 : t_lane;
+        first_ids = seq_idx[(int64_t)b * L + (t > 0 ? t : 0)];
+    }
     // Packed taps are only requested here: everything the run starts with is in flight before
     // the first value is touched (prepare() finishes them).
     constexpr bool WFAST = WM != 0;
@@ -221,7 +196,8 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         }
     };
 
-    auto compute_group = [&](auto checked, int i0, const raw_t (&raw)[U]) {
+    // store = false: a group the masked pass produces; only the window moves on.
+    auto compute_group = [&](auto checked, auto store, int i0, const raw_t (&raw)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             float xv[CH], acc[CH];
@@ -234,7 +210,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
                 a = fmaf(wv[j][W - 1], xv[j], a);
                 acc[j] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
             }
-            if (!decltype(checked)::value || i0 + u <= last)
+            if (decltype(store)::value && (!decltype(checked)::value || i0 + u <= last))
                 store_row(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
 #pragma unroll
             for (int k = 0; k < W - 2; ++k)
@@ -249,10 +225,122 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     using Yes = std::integral_constant<bool, true>;
     static_assert(U >= W - 1, "a group must cover the window");
     raw_t ra[U], rb_[U];
+    // With seq_idx the walk computes every row as if no sub-sequence boundary were near (no
+    // branch, no ids in the hot loop); the groups of U rows whose rows or window are not all of
+    // one non-negative id are redone with masked taps after the walk.  Which groups those are is
+    // found here, with all 64 lanes, a row per lane: lane i holds row i-(W-1) of a stretch of
+    // whole groups and flags it when its id differs from the row before or is negative (rows in
+    // front of the sequence count as id -1 when initial_states are given, as zeros, which no
+    // mask changes, otherwise); group k is redone when a flag falls into its rows or the W-2
+    // rows before them.  Where more than half of the groups are (sub-sequences of a few tokens),
+    // the walk is skipped and the masked pass takes the whole run.
+    const bool full = last >= T - 1;
+    uint32_t redo = 0;
+    bool dense = false;
+    if (HAS_SEQ) {
+        const int n_groups = T / U;
+        if (n_groups > 32) {
+            dense = true;
+        } else {
+            constexpr int kStretch = (kWave - (W - 1)) / U;            // groups per look
+            const int32_t *ids = seq_idx + (int64_t)b * L;
+            const int lane = threadIdx.x & (kWave - 1);
+            const bool init = p.initial_states != nullptr;
+            for (int k0 = 0; k0 < n_groups; k0 += kStretch) {
+                const int t_lane = t0 + k0 * U + lane - (W - 1);       // row of this lane
+                const int t = t_lane > L - 1 ? L - 1 : t_lane;
+                const int id = k0 == 0 ? first_ids : ids[t > 0 ? t : 0];
+                // The id of the row before is the previous lane's (a lane shift, no second load);
+                // lane 0 gets its own id, and its flag belongs to no group's window.
+                const int id_prev = __builtin_amdgcn_update_dpp(id, id, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+                const bool flag = t_lane > L - 1 ? false
+                                : t >= 0 ? (id < 0 || (t > 0 ? id != id_prev : init)) : init;
+                const uint64_t flags = __ballot(flag);
+                for (int k = 0; k < kStretch && k0 + k < n_groups; ++k)
+                    if ((flags >> (k * U + 1)) & ((1ull << (U + W - 2)) - 1)) redo |= 1u << (k0 + k);
+            }
+            int live = last / U + 1;                                   // groups with rows inside the sequence
+            live = live > n_groups ? n_groups : live;
+            redo &= live >= 32 ? ~0u : (1u << live) - 1u;
+            dense = 2 * __builtin_popcount(redo) > live;
+        }
+    }
+    // Rows of a group that will be redone are read with the normal cache policy, so that the
+    // second read finds them in L2; everything else streams through.
+    // The masked pass over one group of U rows: taps masked row by row
+    // (csrc/causal_conv1d_fwd.cu:316-329), padding tokens exactly zero.  masked_request() asks for
+    // the U+W-1 rows and ids the group needs, straight from memory and with no branch between the
+    // loads; masked_finish() computes and stores the group's rows.
+    constexpr int kSpan = U + W - 1;
+    auto masked_request = [&](int i0, raw_t (&rows)[kSpan], int (&sr)[kSpan]) {
+#pragma unroll
+        for (int q = 0; q < kSpan; ++q) {
+            int i = i0 - (W - 1) + q;                  // run-relative row of slot q
+            const bool before = t0 + i < 0;           // in front of the sequence: no data
+            i = i > last ? last : i;
+            i = before ? 0 : i;
+            rows[q] = *reinterpret_cast<const raw_t *>(xrun + (int64_t)i * xs);
+            const int id = seq[i];
+            sr[q] = before ? -1 : id;
+        }
+    };
+    auto masked_finish = [&](int i0, const raw_t (&rows)[kSpan], const int (&sr)[kSpan]) {
+        float xr[kSpan][CH];
+#pragma unroll
+        for (int q = 0; q < kSpan; ++q) P::unpack(rows[q], xr[q]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int cur = sr[W - 1 + u];
+            float acc[CH];
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                float a = bv[j];
+#pragma unroll
+                for (int k = 0; k < W - 1; ++k)
+                    a = fmaf(sr[u + k] == cur ? wv[j][k] : 0.f, xr[u + k][j], a);
+                a = fmaf(wv[j][W - 1], xr[u + W - 1][j], a);
+                if (SILU) a = SCALED ? silu_from_scaled(a) : silu<PRECISE>(a);
+                acc[j] = cur < 0 ? 0.f : a;
+            }
+            if (i0 + u <= last)
+                store_row(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
+        }
+    };
+    auto marked = [&](int i0) { return HAS_SEQ && ((redo >> (i0 / U)) & 1u) != 0; };
+    // A full run does the masked pass of its first marked group up front: the group's rows are
+    // requested here, ahead of the walk's own first rows, so that they cost no memory round trip
+    // of their own (at the end of the walk they would, with nothing left to overlap it), and are
+    // computed and stored while the walk's rows are still in flight.  The walk stores none of the
+    // marked groups; those behind the first are done after it.
+    raw_t early_rows[kSpan];
+    int early_ids[kSpan];
+    const int early = (HAS_SEQ && full && !dense && redo != 0) ? __builtin_ctz(redo) : -1;
+    if (HAS_SEQ) {
+        if (early >= 0) masked_request(early * U, early_rows, early_ids);
+    }
+    if (full && !dense) {
+        if (marked(0)) load_group(No{}, No{}, 0, ra); else load_group(No{}, Yes{}, 0, ra);
+        if (T > 2 * U && !marked(U)) load_group(No{}, Yes{}, U, rb_);
+        else load_group(No{}, No{}, U, rb_);          // the run's last rows: keep them cached
+    }
+    if (!col_ok) return;                              // no cross-lane traffic below
+    auto load_maybe_marked = [&](int i0, raw_t (&raw)[U]) {
+        if (marked(i0)) load_group(No{}, No{}, i0, raw);
+        else load_group(No{}, Yes{}, i0, raw);
+    };
+    auto walk_group = [&](int i0, const raw_t (&raw)[U]) {
+        if (marked(i0)) compute_group(No{}, No{}, i0, raw);
+        else compute_group(No{}, Yes{}, i0, raw);
+    };
+    auto early_masked = [&]() {
+        if (HAS_SEQ) {
+            if (early >= 0) masked_finish(early * U, early_rows, early_ids);
+        }
+    };
     if (dense) {
         // Most groups would be redone: skip the walk, the masked pass below takes the whole run.
         prepare();
-    } else if (last >= T - 1) {
+    } else if (full) {
         // Two register sets in ping-pong: while one group of U rows is computed and stored,
         // the next two groups' loads are in flight, and nothing is copied at the loop edge
         // (a copy would make the compiler wait for every outstanding access).  The first
@@ -260,87 +348,58 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
         // state its back edge leaves (stores A, loads A, stores B, loads B pending), which
         // keeps the compiler's wait counts exact, and no load sits behind an exit test.
         if (T > 2 * U) {
-            load_group(No{}, Yes{}, 0, ra);
-            load_group(No{}, Yes{}, U, rb_);
             prepare();
-            compute_group(No{}, 0, ra);
+            early_masked();
+            walk_group(0, ra);
             int i = 2 * U;
             if (T > 4 * U) {
-                load_group(No{}, Yes{}, 2 * U, ra);
-                compute_group(No{}, U, rb_);
-                load_group(No{}, Yes{}, 3 * U, rb_);
+                load_maybe_marked(2 * U, ra);
+                walk_group(U, rb_);
+                load_maybe_marked(3 * U, rb_);
 #pragma clang loop unroll(disable)
                 for (; i + 4 * U < T; i += 2 * U) {
-                    compute_group(No{}, i, ra);
-                    load_group(No{}, Yes{}, i + 2 * U, ra);
-                    compute_group(No{}, i + U, rb_);
-                    load_group(No{}, Yes{}, i + 3 * U, rb_);
+                    walk_group(i, ra);
+                    load_maybe_marked(i + 2 * U, ra);
+                    walk_group(i + U, rb_);
+                    load_maybe_marked(i + 3 * U, rb_);
                 }
-                compute_group(No{}, i, ra);
-                load_group(No{}, Yes{}, i + 2 * U, ra);
-                compute_group(No{}, i + U, rb_);
+                walk_group(i, ra);
+                load_maybe_marked(i + 2 * U, ra);
+                walk_group(i + U, rb_);
                 i += 2 * U;
             } else {
-                load_group(No{}, Yes{}, 2 * U, ra);
-                compute_group(No{}, U, rb_);
+                load_maybe_marked(2 * U, ra);
+                walk_group(U, rb_);
             }
             load_group(No{}, No{}, i + U, rb_);   // the run's last rows: keep them cached
-            compute_group(No{}, i, ra);
-            compute_group(No{}, i + U, rb_);
+            walk_group(i, ra);
+            walk_group(i + U, rb_);
         } else {
-            load_group(No{}, Yes{}, 0, ra);
-            load_group(No{}, No{}, U, rb_);
             prepare();
-            compute_group(No{}, 0, ra);
-            compute_group(No{}, U, rb_);
+            early_masked();
+            walk_group(0, ra);
+            walk_group(U, rb_);
         }
     } else {
         prepare();
         for (int i = 0; i <= last; i += U) {
             load_group(Yes{}, No{}, i, ra);
-            compute_group(Yes{}, i, ra);
+            if (marked(i)) compute_group(Yes{}, No{}, i, ra);
+            else compute_group(Yes{}, Yes{}, i, ra);
         }
     }
 
     if (HAS_SEQ) {
-        // Rows near a sub-sequence boundary or in padding, one group of U rows per trip:
-        // taps masked row by row (csrc/causal_conv1d_fwd.cu:316-329), padding tokens exactly
-        // zero.  All U+W-1 rows and ids a group needs are requested at once, straight from
-        // memory (they were streamed moments ago), with no branch between the loads; the
-        // results overwrite what the walk stored for these rows.
+        // The marked groups the walk left out (all of the run's groups when the walk was skipped),
+        // one group per trip.
         const int live_rows = last + 1 < T ? last + 1 : T;
 #pragma clang loop unroll(disable)
         for (int i0 = 0; i0 < live_rows; i0 += U) {
-            if (!dense && !((redo >> (i0 / U)) & 1u)) continue;
-            float xr[U + W - 1][CH];
-            int sr[U + W - 1];
-#pragma unroll
-            for (int q = 0; q < U + W - 1; ++q) {
-                int i = i0 - (W - 1) + q;              // run-relative row of slot q
-                const bool before = t0 + i < 0;       // in front of the sequence: no data
-                i = i > last ? last : i;
-                i = before ? 0 : i;
-                P::unpack(*reinterpret_cast<const raw_t *>(xrun + (int64_t)i * xs), xr[q]);
-                const int id = seq[i];
-                sr[q] = before ? -1 : id;
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int cur = sr[W - 1 + u];
-                float acc[CH];
-#pragma unroll
-                for (int j = 0; j < CH; ++j) {
-                    float a = bv[j];
-#pragma unroll
-                    for (int k = 0; k < W - 1; ++k)
-                        a = fmaf(sr[u + k] == cur ? wv[j][k] : 0.f, xr[u + k][j], a);
-                    a = fmaf(wv[j][W - 1], xr[u + W - 1][j], a);
-                    if (SILU) a = SCALED ? silu_from_scaled(a) : silu<PRECISE>(a);
-                    acc[j] = cur < 0 ? 0.f : a;
-                }
-                if (i0 + u <= last)
-                    store_row(P::pack(acc), reinterpret_cast<raw_t *>(orun + (uint32_t)(i0 + u) * os));
-            }
+            if (!dense && (!marked(i0) || i0 == early * U)) continue;
+            raw_t rows[kSpan];
+            int sr[kSpan];
+            masked_request(i0, rows, sr);
+            masked_finish(i0, rows, sr);
         }
     }
 
@@ -458,31 +517,48 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     g.total = (uint32_t)total;
     const uint32_t blocks = (uint32_t)((total + kBlock / kWave - 1) / (kBlock / kWave));
     // Workgroup order: an XCD takes chunks of `chunk_runs` consecutive runs (all their column
-    // blocks), the 8 XCDs take 8 neighbouring chunks at a time.
-    // Against one contiguous slice of the launch per XCD (8 streams far apart in memory, each with
-    // its own address translations to fetch), chunks of 8 runs measured, warm / on rotating buffers
-    // that do not fit the translation caches: (8, 5376, 2048) bf16 55.6 / 65.1 -> 55.8 / 63.9 us,
-    // (4, 4096, 4096) 43.9 / 51.8 -> 43.5 / 50.0 us, (16, 2048, 2048) 46.3 / 56.2 -> 43.7 / 49.5 us.  Only the
-    // first run of a chunk finds its halo rows in another XCD's L2.  Launches of fewer than eight
-    // chunks per XCD take chunks of 4 runs, or else contiguous slices ((2, 8192, 2048): 22.9 us in
-    // slices, 25.9 us in 32 chunks).
+    // blocks), the 8 XCDs take 8 neighbouring chunks at a time.  Inside a chunk a run finds the halo
+    // rows it shares with the run above in its own XCD's L2; across XCDs the chip walks through
+    // memory as one front instead of eight far-apart streams, which is what counts on buffers that
+    // are not already in the caches and translation caches (every layer of a model).  Chunk sizes
+    // are measured, warm / on rotating buffer sets of 2 GB, bf16, in us:
+    //   row of 42 wavefronts (8, 5376, 2048): slices 54.2 / 62.6, chunks of 2 runs 54.4 / 60.8, 4 runs
+    //     53.6 / 60.9, 8 runs 53.2 / 61.5, 16 runs 54.5 / 63.8, hardware order 55.7 / 60.3; the same
+    //     picture at (16, 5376, 1024), (32, 5376, 512), (1, 5376, 16384), in fp16 and in fp32
+    //   80 wavefronts (2, 10240, 4096): slices 52.9 / 61.2, 2 runs 52.0 / 59.0, 4 runs 53.8 / 61.3
+    //   64 wavefronts (4, 8192, 2048): slices 41.8 / 48.0, 4 runs 43.7 / 49.9, 16 runs 42.0 / 47.7
+    //   32 wavefronts (8, 4096, 2048): slices 42.4 / 50.8, 8 runs 42.7 / 50.6, 16 runs 41.8 / 48.3
+    //   16 wavefronts (16, 2048, 2048): slices 44.5 / 54.8, 8 runs 42.0 / 47.7, 16 runs 42.0 / 48.1
+    // (row strides that are large powers of two want the XCDs further apart).  Launches of fewer
+    // than eight chunks per XCD take smaller chunks, or else contiguous slices ((2, 8192, 2048):
+    // 22.9 us in slices, 25.9 us in 32 chunks).
     int chunk_runs = tunables().fwd_cl_chunk_runs;
-    // Rows wider than 32 wavefronts gain nothing from chunks, and the headline shape (42 wavefronts
-    // a row, one batch entry per XCD) measured 55.3-55.5 us in slices against 56.7-57.0 us in chunks.
-    if (chunk_runs == 0 && g.waves_per_row > 32) chunk_runs = -1;
-    if (chunk_runs == 0 && p.x_dtype == CC1D_F32) {
-        // fp32 rows (twice the bytes, fewer wavefronts per CU) measured best in chunks of 16 runs, from
-        // four chunks per XCD on: (4, 2048, 4096) 42.5 us in slices, 46.6 in chunks of 8, 41.8 in chunks of
-        // 16 (cold 48.1 / 55.5 / 48.3); (16, 2048, 2048) 79.6 / 81.5 / 78.0 us (cold 98 / 102 / 92.6).
-        chunk_runs = 16;
-        if ((int64_t)blocks < (int64_t)4 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = -1;
-    } else if (chunk_runs == 0) {
-        chunk_runs = 8;
-        if ((int64_t)blocks < (int64_t)8 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = 4;
-        if ((int64_t)blocks < (int64_t)8 * kXcds * (chunk_runs / 4) * g.waves_per_row) chunk_runs = -1;
+    if (chunk_runs == 0) {
+        const int64_t wpr = g.waves_per_row;
+        if (p.x_dtype == CC1D_F32 && wpr <= 32) {
+            // fp32 rows (twice the bytes, fewer wavefronts per CU) measured best in chunks of 16 runs,
+            // from four chunks per XCD on: (4, 2048, 4096) 42.5 us in slices, 46.6 in chunks of 8, 41.8 in
+            // chunks of 16 (cold 48.1 / 55.5 / 48.3); (16, 2048, 2048) 79.6 / 81.5 / 78.0 us (cold 98 / 102 / 92.6).
+            chunk_runs = 16;
+            if ((int64_t)blocks < 4 * kXcds * (chunk_runs / 4) * wpr) chunk_runs = -1;
+        } else {
+            // chunks per XCD the launch gives at a chunk size
+            auto chunks_per_xcd = [&](int runs) { return (int64_t)blocks * 4 / ((int64_t)kXcds * runs * wpr); };
+            if (wpr > 64) chunk_runs = chunks_per_xcd(2) >= 8 ? 2 : -1;
+            else if (wpr > 48) chunk_runs = chunks_per_xcd(16) >= 4 ? 16 : -1;
+            else if (wpr > 32) chunk_runs = chunks_per_xcd(4) >= 8 ? 4 : -1;
+            else {
+                chunk_runs = wpr > 16 && chunks_per_xcd(16) >= 4 ? 16 : 8;
+                if (chunk_runs == 8 && chunks_per_xcd(8) < 8) chunk_runs = 4;
+                if (chunk_runs == 4 && chunks_per_xcd(4) < 8) chunk_runs = -1;
+            }
+        }
     }
-    g.blocks_per_chunk = chunk_runs <= 0 ? 0u : (uint32_t)(chunk_runs / 4 > 0 ? chunk_runs / 4 : 1) * g.waves_per_row;
-    if (chunk_runs < -1) g.blocks_per_chunk = (uint32_t)(-chunk_runs);   // sweeps: chunks of so many workgroups
+    // chunk_runs > 0: chunks of that many runs (a run is waves_per_row wavefronts, a workgroup four of
+    // them); < -1: chunks of -chunk_runs - 1 workgroups (-2: one workgroup, which is the hardware's own
+    // round-robin order); -1: one contiguous slice per XCD.
+    g.blocks_per_chunk = chunk_runs > 0 ? (uint32_t)(((int64_t)chunk_runs * g.waves_per_row + 3) / 4)
+                         : chunk_runs < -1 ? (uint32_t)(-chunk_runs - 1) : 0u;
     g.blocks_per_xcd = (blocks + kXcds - 1) / kXcds;
     if (g.blocks_per_chunk != 0)
         g.blocks_per_xcd = (g.blocks_per_xcd + g.blocks_per_chunk - 1) / g.blocks_per_chunk * g.blocks_per_chunk;

@@ -265,11 +265,13 @@ int cc1d_hip_runtime_path(char *path, size_t size);
  *   "fwd_cl_rows"   rows of seqlen walked by one lane of the channel-last forward
  *   "fwd_cl_half_vec" -1 = the channel-last forward reads its taps with the general loader even
  *                   when they are packed
- *   "fwd_cl_chunk_runs" consecutive runs an XCD takes before the next XCD's in the channel-last
- *                   forward's workgroup order (a multiple of 4; -1 = one contiguous slice per XCD;
- *                   -n, n > 1 = chunks of n workgroups)
+ *   "fwd_cl_chunk_runs" workgroup order of the channel-last forward: n > 0 = an XCD takes chunks of n
+ *                   consecutive runs, the 8 XCDs side by side on 8 neighbouring chunks; -1 = one
+ *                   contiguous slice of the launch per XCD; -n, n > 1 = chunks of n-1 workgroups
+ *                   (-2: single workgroups, the hardware's own round-robin order)
  *   "bwd_cl_rows"   same for the channel-last backward
- *   "bwd_cl_chunk_runs" as "fwd_cl_chunk_runs", for the channel-last backward
+ *   "bwd_cl_chunk_runs" the same for the channel-last backward, whose workgroups take 4 runs each:
+ *                   n >= 4 = chunks of n / 4 workgroup rows; -1 = one contiguous slice per XCD
  *   "fwd_cf_vecs"   16-byte vectors per wave segment in the channel-first forward
  *   "bwd_cf_parts"  partitions of (batch x seqlen) per channel in the channel-first backward
  *   "launch_limit_shift" n: one launch holds at most 2^(31-n) threads instead of 2^31 (n <= 24), so
