@@ -67,7 +67,18 @@ struct RowCtx {
     int64_t xrow, drow;
     float wv[W];
     float bias_v;
+    float wvs[W], bias_s;         // taps and bias times -log2(e), for the activation's derivative
     bool silu_on;
+
+    __device__ __forceinline__ void scale_taps() {
+#pragma unroll
+        for (int w = 0; w < W; ++w) wvs[w] = wv[w] * kSiluPrescale;
+        bias_s = bias_v * kSiluPrescale;
+    }
+    // act'(z) at the position whose window is xwin[0 .. W)
+    __device__ __forceinline__ float act_grad(const float *xwin) const {
+        return silu_grad_of_window<W, Elem<DT>::kPreciseAct>(wv, bias_v, wvs, bias_s, xwin);
+    }
 
     // xpad[t] for t < L, raw bits
     __device__ __forceinline__ typename Elem<DT>::type x_raw_at(int t) const {
@@ -122,12 +133,7 @@ struct RowCtx {
         for (int k = 0; k < N; ++k) {
             const int q = t0 + k;
             float gk = q >= 0 && q < L ? Elem<DT>::to_float(draw[k]) : 0.f;
-            if (silu_on) {
-                float z = bias_v;
-#pragma unroll
-                for (int w = 0; w < W; ++w) z = fmaf(wv[w], xp[k + w], z);
-                gk *= silu_grad<Elem<DT>::kPreciseAct>(z);
-            }
+            if (silu_on) gk *= act_grad(&xp[k]);
             gv[k] = gk;
         }
     }
@@ -136,10 +142,10 @@ struct RowCtx {
         if (t < 0 || t >= p.seqlen) return 0.f;
         float gv = ld_elem<DT>(p.dout, drow + t);
         if (silu_on) {
-            float z = bias_v;
+            float xwin[W];
 #pragma unroll
-            for (int w = 0; w < W; ++w) z = fmaf(wv[w], x_at(t - (W - 1) + w), z);
-            gv *= silu_grad<Elem<DT>::kPreciseAct>(z);
+            for (int w = 0; w < W; ++w) xwin[w] = x_at(t - (W - 1) + w);
+            gv *= act_grad(xwin);
         }
         return gv;
     }
@@ -167,6 +173,7 @@ bwd_channelfirst_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__res
     for (int w = 0; w < W; ++w)
         rc.wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
     rc.bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+    rc.scale_taps();
 
     float dW[W], dB = 0.f;
 #pragma unroll
@@ -264,10 +271,7 @@ bwd_channelfirst_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float *__res
                 if (rc.silu_on) {
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        float z = rc.bias_v;
-#pragma unroll
-                        for (int w = 0; w < W; ++w) z = fmaf(rc.wv[w], xx[e + w], z);
-                        gf[e] *= silu_grad<PRECISE>(z);
+                        gf[e] *= rc.act_grad(&xx[e]);
                     }
                 }
 
@@ -385,6 +389,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
     for (int w = 0; w < W; ++w)
         rc.wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
     rc.bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+    rc.scale_taps();
 
     float dW[W], dB = 0.f;
 #pragma unroll
@@ -524,10 +529,7 @@ bwd_channelfirst_stream_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float
             if (rc.silu_on) {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    float z = rc.bias_v;
-#pragma unroll
-                    for (int w = 0; w < W; ++w) z = fmaf(rc.wv[w], xx[e + w], z);
-                    gf[e] *= silu_grad<PRECISE>(z);
+                    gf[e] *= rc.act_grad(&xx[e]);
                 }
             }
             // gg[i] = g at position tf+i, i in [0, VEC+W-1)
@@ -688,6 +690,10 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
     for (int w = 0; w < W; ++w)
         wv[w] = ld_weight(p.weight, p.w_dtype, (int64_t)c * p.w_stride_c + w * p.w_stride_w);
     bias_v = p.bias == nullptr ? 0.f : ld_weight(p.bias, p.w_dtype, c);
+    float wvs[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w) wvs[w] = wv[w] * kSiluPrescale;
+    const float bias_s = bias_v * kSiluPrescale;
 
     float dW[W], dB = 0.f;
 #pragma unroll
@@ -752,10 +758,7 @@ bwd_channelfirst_short_kernel(const cc1d_bwd_params p, const BwdCfGeom g, float 
         if (silu_on) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                float z = bias_v;
-#pragma unroll
-                for (int w = 0; w < W; ++w) z = fmaf(wv[w], xx[e + w], z);
-                gf[e] *= silu_grad<PRECISE>(z);
+                gf[e] *= silu_grad_of_window<W, PRECISE>(wv, bias_v, wvs, bias_s, &xx[e]);
             }
         }
 

@@ -67,6 +67,7 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
     using P = Pack<DT, CH>;
     using raw_t = typename P::raw_t;
     constexpr bool PRECISE = E::kPreciseAct;
+    constexpr bool SCALED = SILU && !PRECISE;         // taps, bias and g carry the factor of the SiLU exponent
 
     const int c0 = (int)col * CH;
     const int L = p.seqlen;
@@ -113,7 +114,7 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
                 for (int k = 0; k < W - 1; ++k)
                     z = fmaf((!MASKED || idwin[k] == cur) ? xwin[k][j] : 0.f, wv[j][k], z);
                 z = fmaf(wv[j][W - 1], xv[j], z);
-                gv[j] *= silu_grad<PRECISE>(z);
+                gv[j] *= SCALED ? silu_grad_from_scaled_over_c(z) : silu_grad<PRECISE>(z);
             }
         }
         if (MASKED) {
@@ -166,6 +167,17 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
     auto fill_windows = [&]() __attribute__((always_inline)) {
         if (WM != 0) taps.finish(p.bias != nullptr, wv, bv);
         else any_taps.finish(p.w_dtype, p.bias != nullptr, wv, bv);
+        // With SiLU the lane keeps only c w and c bias, c = -log2(e): the sums over the taps are
+        // then the exponent the activation's derivative needs, g is carried as g / c, dx comes out
+        // unscaled (c w times g / c), and the kernel multiplies its dweight / dbias sums by c once.
+        if (SCALED) {
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                bv[j] *= kSiluPrescale;
+#pragma unroll
+                for (int k = 0; k < W; ++k) wv[j][k] *= kSiluPrescale;
+            }
+        }
         float xh[2 * (W - 1)][CH];
 #pragma unroll
         for (int q = 0; q < 2 * (W - 1); ++q) P::unpack(xh_raw[q], xh[q]);
@@ -421,6 +433,7 @@ bwd_channellast_kernel(const cc1d_bwd_params p, const BwdClGeom g, float *__rest
                 float v = w < W ? dW[j][w] : dB[j];
 #pragma unroll
                 for (int r = 0; r < kRunsPerBlock - 1; ++r) v += partial[r][w * CH + j][lane];
+                if (SILU && !Elem<DT>::kPreciseAct) v *= kSiluPrescale;     // the runs summed g / c
                 o[j] = bitcast<uint32_t>(v);
             }
             *reinterpret_cast<typename RawBytes<CH * 4>::type *>(dst + (int64_t)w * p.dim) = o;

@@ -452,6 +452,39 @@ __device__ __forceinline__ float silu_grad(float z) {
     const float s = sigmoid<PRECISE>(z);
     return s * (1.0f + z * (1.0f - s));
 }
+// The same derivative given y = -log2(e) z, the pre-activation formed with taps and bias that
+// carry that factor (one multiply per element less than forming z and scaling it):
+//   s = 1 / (1 + 2^y),   z (1 - s) = y k (1 - s) with k = -ln 2,   k (1 - s) = k - k s.
+__device__ __forceinline__ float silu_grad_from_scaled(float y) {
+    constexpr float k = -0.6931471805599453f;
+    const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(y));
+    return s * fmaf(y, fmaf(-k, s, k), 1.0f);
+}
+// The derivative divided by c = -log2(e), for kernels that keep only the prescaled taps c w:
+// with g' = dout act'(z) / c, dx = sum (c w) g' is the true dx, and the sums of g' x and of g'
+// are dweight / c and dbias / c (multiplied by c once, at the end).  1 / c = -ln 2 = k.
+__device__ __forceinline__ float silu_grad_from_scaled_over_c(float y) {
+    constexpr float k = -0.6931471805599453f, kk = 0.4804530139182014f;   // kk = k^2
+    const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(y));
+    return s * fmaf(y, fmaf(-kk, s, kk), k);
+}
+// d silu / dz at z = bias + sum_w wv[w] xwin[w].  The fast variant takes the taps and bias
+// prescaled by -log2(e) (wvs, bias_s); the precise one the plain ones.
+template <int W, bool PRECISE>
+__device__ __forceinline__ float silu_grad_of_window(const float (&wv)[W], float bias_v, const float (&wvs)[W],
+                                                     float bias_s, const float *xwin) {
+    if constexpr (PRECISE) {
+        float z = bias_v;
+#pragma unroll
+        for (int w = 0; w < W; ++w) z = fmaf(wv[w], xwin[w], z);
+        return silu_grad<true>(z);
+    } else {
+        float y = bias_s;
+#pragma unroll
+        for (int w = 0; w < W; ++w) y = fmaf(wvs[w], xwin[w], y);
+        return silu_grad_from_scaled(y);
+    }
+}
 
 template <int DT, int CH>
 struct alignas(CH * Elem<DT>::kBytes) RawElems {
