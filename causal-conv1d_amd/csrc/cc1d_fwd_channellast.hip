@@ -237,6 +237,7 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     const bool full = last >= T - 1;
     uint32_t redo = 0;
     bool dense = false;
+    auto look_at_ids = [&]() __attribute__((always_inline)) {
     if (HAS_SEQ) {
         const int n_groups = T / U;
         if (n_groups > 32) {
@@ -265,8 +266,12 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
             dense = 2 * __builtin_popcount(redo) > live;
         }
     }
-    // Rows of a group that will be redone are read with the normal cache policy, so that the
-    // second read finds them in L2; everything else streams through.
+    };
+    // The look comes before the run's first rows are requested.  Requesting the rows first and
+    // looking at the ids while they are in flight (the ids, requested before everything else, are
+    // back long before them) takes the look out of the wavefront's critical path, and measured
+    // 3.4 us slower on warm buffers (56.1 against 52.7 us) for 1.3 us gained on cold ones.
+    look_at_ids();
     // The masked pass over one group of U rows: taps masked row by row
     // (csrc/causal_conv1d_fwd.cu:316-329), padding tokens exactly zero.  masked_request() asks for
     // the U+W-1 rows and ids the group needs, straight from memory and with no branch between the
@@ -318,6 +323,8 @@ fwd_channellast_kernel(const cc1d_fwd_params p, const FwdClGeom g, const int32_t
     if (HAS_SEQ) {
         if (early >= 0) masked_request(early * U, early_rows, early_ids);
     }
+    // Rows of a group that will be redone are read with the normal cache policy, so that the
+    // second read finds them in L2; everything else streams through.
     if (full && !dense) {
         if (marked(0)) load_group(No{}, No{}, 0, ra); else load_group(No{}, Yes{}, 0, ra);
         if (T > 2 * U && !marked(U)) load_group(No{}, Yes{}, U, rb_);
