@@ -476,18 +476,32 @@ int launch_lanes(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTail 
 
 // Rows walked by one lane.  Longer runs amortise the per-run start-up (taps, halo); shorter
 // runs put more wavefronts in flight, which is what keeps HBM busy while other waves
-// compute, and spread the work more evenly over the CUs.  32 rows measured best at the
-// prefill shape (8 x 2048 rows x 5376 channels); short sequences take what they have.
+// compute, and spread the work more evenly over the CUs, and on buffers no cache holds they
+// keep the chip's accesses closer together in memory.  32 rows measured best on warm buffers at
+// the prefill shape (8 x 2048 rows x 5376 channels) without seq_idx; short sequences take what they have.
 // A launch that fills the chip's wavefront slots (256 CUs x 4 SIMDs x `waves_per_simd`) less than
 // 0.6 times over with 32-row runs is bound by the length of a wavefront's own chain of loads,
 // not by bandwidth, and takes 16-row runs: 3.7 against 4.6 us at (1, 5376, 64) bf16, 5.5 against
 // 6.2 us at (1, 5376, 1024), 8.6 against 9.5 us at (1, 5376, 1024) fp32; from about one fill
-// upwards 32 rows are as good or better.
-static int choose_rows_per_run(int seqlen, int64_t row_bytes, int64_t waves_per_row_of_runs, int waves_per_simd) {
+// upwards 32 rows are as good or better for 16-bit data.
+// fp32 rows (8-byte lanes, three wavefronts per SIMD) take 16-row runs at every size: warm / on
+// rotating buffer sets, 16 against 32 rows, (4, 2048, 4096) 42.2 / 46.9 against 43.4 / 48.8 us,
+// (16, 2048, 2048) 78.9 / 89.1 against 79.6 / 94.4, (8, 5376, 2048) 103.5 / 117.9 against 103.1 / 121.6,
+// the same with seq_idx 115.8 / 118.0 against 120.9 / 125.0, (64, 768, 1024) 61.1 / 69.3 against
+// 62.2 / 72.6; (4, 8192, 2048) is the one shape of fourteen that lost on rotating sets (90.5 against 88.0).
+// bf16 / fp16 with seq_idx take 16-row runs as well: (8, 5376, 2048) 52.5 / 61.4 against 52.5 / 63.3 us,
+// (8, 4096, 2048) 40.0 / 47.5 against 40.9 / 50.2, (16, 2048, 2048) 40.4 / 47.3 against 41.2 / 50.2,
+// (2, 10240, 4096) 51.6 / 58.9 against 50.7 / 61.2, (8, 6144, 2048) 59.6 / 69.4 against 59.5 / 73.8.
+// Without seq_idx 16-row runs gain 0.3 to 1.7 us on rotating sets and lose 1 to 2.5 us on warm ones
+// ((8, 5376, 2048) 55.2 / 59.2 against 53.6 / 60.9): they keep 32 rows.
+// (A copy kernel that walks the prefill tensor the same way, no arithmetic, takes 59.1 us on
+// rotating sets in 32-row runs and 56.0 us in 16-row runs, a plain linear copy 55.6 us.)
+static int choose_rows_per_run(int seqlen, int64_t row_bytes, int64_t waves_per_row_of_runs, int waves_per_simd,
+                               bool short_runs) {
     constexpr int U = 2 * CC1D_FWD_CL_UNROLL;         // the walk is unrolled over two groups
     int T = tunables().fwd_cl_rows;
     if (T <= 0) {
-        T = 32;
+        T = short_runs ? 16 : 32;
         const int64_t waves32 = waves_per_row_of_runs * ((seqlen + 31) / 32);
         if (10 * waves32 <= 6 * (int64_t)(256 * 4) * waves_per_simd) T = 16;
     }
@@ -516,7 +530,8 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
     g.waves_per_row = (uint32_t)((g.n_colgroups + kWave - 1) / kWave);
     g.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * elem_bytes(p.x_dtype), (int64_t)p.batch * g.waves_per_row,
-                                         p.x_dtype == CC1D_F32 ? CC1D_FWD_CL_OCC8 : CC1D_FWD_CL_OCC4);
+                                         p.x_dtype == CC1D_F32 ? CC1D_FWD_CL_OCC8 : CC1D_FWD_CL_OCC4,
+                                         p.x_dtype == CC1D_F32 || p.seq_idx != nullptr);
     if (g.rows_per_run == 0) return CC1D_ERR_TOO_LARGE;
     g.n_runs = (p.seqlen + g.rows_per_run - 1) / g.rows_per_run;
     const int64_t total = (int64_t)p.batch * g.n_runs * g.waves_per_row;
