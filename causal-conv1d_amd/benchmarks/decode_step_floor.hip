@@ -26,6 +26,8 @@ using namespace cc1d;
 __global__ void __launch_bounds__(256) empty_kernel(const StepArgs a) { if (a.batch < 0) *(int *)a.out = 0; }
 
 // Same footprint as the linear step, no arithmetic: per (row, colgroup) read 4 x 8 bytes, write 4 x 8 bytes.
+// NT: the state rows with the non-temporal policy, as the step kernel reads and writes them.
+template <bool NT>
 __global__ void __launch_bounds__(256) copy_kernel(const StepArgs a) {
     using raw_t = u32x2;
     const uint32_t lane = threadIdx.x & 63;
@@ -38,13 +40,20 @@ __global__ void __launch_bounds__(256) copy_kernel(const StepArgs a) {
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
 #pragma unroll
-        for (int i = 0; i < 3; ++i) v[r][i] = *reinterpret_cast<const raw_t *>(sb + (int64_t)(b0 + r) * a.state_stride_b + c0 + (int64_t)i * a.state_stride_l);
+        for (int i = 0; i < 3; ++i) {
+            const raw_t *src = reinterpret_cast<const raw_t *>(sb + (int64_t)(b0 + r) * a.state_stride_b + c0 + (int64_t)i * a.state_stride_l);
+            v[r][i] = NT ? __builtin_nontemporal_load(src) : *src;
+        }
         v[r][3] = *reinterpret_cast<const raw_t *>(xb + (int64_t)(b0 + r) * a.x_stride_b + c0);
     }
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
 #pragma unroll
-        for (int i = 0; i < 3; ++i) *reinterpret_cast<raw_t *>(sb + (int64_t)(b0 + r) * a.state_stride_b + c0 + (int64_t)i * a.state_stride_l) = v[r][(i + 1) & 3];
+        for (int i = 0; i < 3; ++i) {
+            raw_t *dst = reinterpret_cast<raw_t *>(sb + (int64_t)(b0 + r) * a.state_stride_b + c0 + (int64_t)i * a.state_stride_l);
+            if (NT) __builtin_nontemporal_store(v[r][(i + 1) & 3], dst);
+            else *dst = v[r][(i + 1) & 3];
+        }
         *reinterpret_cast<raw_t *>(ob + (int64_t)(b0 + r) * a.out_stride_b + c0) = v[r][0];
     }
 }
@@ -128,7 +137,8 @@ int main(int argc, char **argv) {
         std::vector<Variant> vs;
         vs.push_back({"library launch_update", [](const StepArgs &, const cc1d_update_params &p, hipStream_t s, int) { launch_update(p, s); }});
         vs.push_back({"empty kernel, same grid", [](const StepArgs &a, const cc1d_update_params &, hipStream_t s, int) { hipLaunchKernelGGL(empty_kernel, dim3(21, 32), dim3(256), 0, s, a); }});
-        vs.push_back({"copy kernel, linear footprint", [](const StepArgs &a, const cc1d_update_params &, hipStream_t s, int) { hipLaunchKernelGGL(copy_kernel, dim3(21, 32), dim3(256), 0, s, a); }});
+        vs.push_back({"copy kernel, linear footprint", [](const StepArgs &a, const cc1d_update_params &, hipStream_t s, int) { hipLaunchKernelGGL(copy_kernel<false>, dim3(21, 32), dim3(256), 0, s, a); }});
+        vs.push_back({"copy kernel, state rows non-temporal", [](const StepArgs &a, const cc1d_update_params &, hipStream_t s, int) { hipLaunchKernelGGL(copy_kernel<true>, dim3(21, 32), dim3(256), 0, s, a); }});
 #define COPYT(CHB, R) vs.push_back({"copy " #CHB " ch/lane R=" #R, [](const StepArgs &a, const cc1d_update_params &, hipStream_t s, int) { \
             const uint32_t ncg = a.n_colgroups * 4 / CHB; \
             hipLaunchKernelGGL((copy_kernel_t<CHB, R>), dim3((ncg + 63) / 64, a.batch / (4 * R)), dim3(256), 0, s, a); }})

@@ -239,6 +239,20 @@ struct WorkgroupTaps {
     }
 };
 
+// conv_state rows are read and written with the non-temporal policy: a step touches every state
+// row of its layer exactly once, and by the time the same layer's next step comes round a model's
+// other layers have been through the caches.  At (256, 5376) bf16, width 4, plain / non-temporal,
+// us per launch: state (.., 3) shifted in place 4.59 / 4.17-4.37 on one set of buffers and 6.80 / 5.58
+// over 40 rotating sets; ring buffer (.., 8) 4.13 / 4.22 and 5.89 / 4.99.  (Loads alone: 4.60 / 5.98 and
+// 4.17 / 5.37; stores alone: 4.52 / 6.76 and 3.96 / 5.58.)  x and out keep the plain policy: the
+// non-temporal one measured 0.1 us slower for them.  So do the rows in front of the window that a
+// state longer than the window shifts along in place: (.., 8) shifted, 7.5 us on one set with the
+// plain policy for them against 10.8 us with the non-temporal one.
+template <typename V>
+__device__ __forceinline__ V ld_state(const V *p) { return __builtin_nontemporal_load(p); }
+template <typename V>
+__device__ __forceinline__ void st_state(V *p, const V &v) { __builtin_nontemporal_store(v, p); }
+
 // Decode step, one token.  A workgroup takes 64 adjacent column groups (one per lane) of
 // 4 x R batch entries (R per wavefront): grid x = blocks of 64 column groups, y = batch / (4 R).
 // The taps come through WorkgroupTaps.
@@ -289,7 +303,7 @@ update_step_kernel(const StepArgs a) {
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) {
             const int l = CIRC ? wrap(cs - (W - 1) + i, S) : S - (W - 1) + i;
-            rw[r][i] = *reinterpret_cast<const raw_t *>(sbase + soff[r] + (int64_t)l * a.state_stride_l);
+            rw[r][i] = ld_state(reinterpret_cast<const raw_t *>(sbase + soff[r] + (int64_t)l * a.state_stride_l));
         }
         xr[r] = *reinterpret_cast<const raw_t *>(xb + (int64_t)bb * a.x_stride_b + c0);
     }
@@ -313,7 +327,7 @@ update_step_kernel(const StepArgs a) {
         }
         T *st = sbase + soff[r];
         if (CIRC) {
-            *reinterpret_cast<raw_t *>(st + (int64_t)wpos[r] * a.state_stride_l) = xr[r];
+            st_state(reinterpret_cast<raw_t *>(st + (int64_t)wpos[r] * a.state_stride_l), xr[r]);
         } else {
             // new_state = concat(state, x)[-S:]: rows in front of the window move up by one
             // (reads run ahead of writes), the window rows come straight from registers.
@@ -321,11 +335,11 @@ update_step_kernel(const StepArgs a) {
             for (int j = 0; j + 1 < head; ++j)
                 *reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l) =
                     *reinterpret_cast<const raw_t *>(st + (int64_t)(j + 1) * a.state_stride_l);
-            if (head > 0) *reinterpret_cast<raw_t *>(st + (int64_t)(head - 1) * a.state_stride_l) = rw[r][0];
+            if (head > 0) st_state(reinterpret_cast<raw_t *>(st + (int64_t)(head - 1) * a.state_stride_l), rw[r][0]);
 #pragma unroll
             for (int k = 0; k < W - 2; ++k)
-                *reinterpret_cast<raw_t *>(st + (int64_t)(head + k) * a.state_stride_l) = rw[r][k + 1];
-            *reinterpret_cast<raw_t *>(st + (int64_t)(S - 1) * a.state_stride_l) = xr[r];
+                st_state(reinterpret_cast<raw_t *>(st + (int64_t)(head + k) * a.state_stride_l), rw[r][k + 1]);
+            st_state(reinterpret_cast<raw_t *>(st + (int64_t)(S - 1) * a.state_stride_l), xr[r]);
         }
         float xv[CH], acc[CH], f[W - 1][CH];
 #pragma unroll
@@ -396,7 +410,7 @@ update_tokens_kernel(const TokensArgs ta) {
 #pragma unroll
     for (int i = 0; i < W - 1; ++i) {
         const int l = CIRC ? wrap(cs - (W - 1) + i, S) : S - (W - 1) + i;
-        rw[i] = *reinterpret_cast<const raw_t *>(st + (int64_t)l * a.state_stride_l);
+        rw[i] = ld_state(reinterpret_cast<const raw_t *>(st + (int64_t)l * a.state_stride_l));
     }
 #pragma unroll
     for (int i = 0; i < kMaxTokens; ++i) {
@@ -419,7 +433,7 @@ update_tokens_kernel(const TokensArgs ta) {
 #pragma unroll
         for (int i = 0; i < kMaxTokens; ++i) {
             if (i < L) {
-                *reinterpret_cast<raw_t *>(st + (int64_t)wpos * a.state_stride_l) = xr[i];
+                st_state(reinterpret_cast<raw_t *>(st + (int64_t)wpos * a.state_stride_l), xr[i]);
                 wpos = wpos + 1 == S ? 0 : wpos + 1;
             }
         }
@@ -433,12 +447,12 @@ update_tokens_kernel(const TokensArgs ta) {
 #pragma unroll
         for (int k = 0; k < W - 1; ++k) {
             const int j = head + k - L;
-            if (j >= 0) *reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l) = rw[k];
+            if (j >= 0) st_state(reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l), rw[k]);
         }
 #pragma unroll
         for (int i = 0; i < kMaxTokens; ++i) {
             const int j = S - L + i;
-            if (i < L && j >= 0) *reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l) = xr[i];
+            if (i < L && j >= 0) st_state(reinterpret_cast<raw_t *>(st + (int64_t)j * a.state_stride_l), xr[i]);
         }
     }
 
