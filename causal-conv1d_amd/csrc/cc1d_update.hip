@@ -554,6 +554,99 @@ update_generic_kernel(const cc1d_update_params p, const uint32_t total) {
     }
 }
 
+// Decode step, one token, for conv_state with unit stride along state_len: the (batch, dim,
+// state_len) contiguous cache that mamba_ssm's Mamba block allocates (state_len = d_conv), where a
+// channel's whole state is state_len consecutive elements.  A lane moves one 16-byte vector of
+// it: CH = 16 / (state_len * element size) adjacent channels (two channels of four bf16 states,
+// one of four fp32 states ...), loaded once, shifted by one position in registers
+// (new_state = concat(state, x)[-state_len:], csrc/causal_conv1d_update.cu:72-84,95-98) and stored
+// once; x, out and the taps of those channels are the lane's other accesses, and the taps serve R
+// batch entries.  Grid: x = groups of CH channels / 256, y = batch / R (no division per lane).  Same arithmetic, in the same order,
+// as the other update kernels; the state moves as raw bits.  (256, 5120) bf16, state_len 4, on the same
+// buffers every call / on 40 sets of buffers in turn: 12.4 / 14.6 us with one element access per
+// state position, 4.7 / 6.0-6.3 us here with R = 2 (5.1 / 7.6-7.8 with R = 1, 4.8 / 7.1 with R = 4),
+// 4.7 / 6.1 us for the cache with unit stride along dim.
+template <int DT, int W, int CH, bool SILU, bool PACKED16, int R>
+__global__ void __launch_bounds__(kBlock)
+update_rowstate_kernel(const cc1d_update_params p, const uint32_t n_groups, const int w_contiguous_f32) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    constexpr bool PRECISE = E::kPreciseAct;
+    constexpr int S = 16 / (CH * E::kBytes);          // state_len
+    static_assert(S * CH * E::kBytes == 16 && S >= W - 1, "one 16-byte vector holds CH whole states");
+
+    const uint32_t cg = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
+    if (cg >= n_groups) return;
+    const int c0 = (int)cg * CH;
+    const int b0 = (int)blockIdx.y * R;               // the lane's R batch entries share its taps
+
+    u32x4 *sp[R];
+    u32x4 raw[R];
+    T xe[R][CH];
+    bool live[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int b = b0 + r;
+        live[r] = false;
+        if (b >= p.batch) continue;
+        const int srow = p.conv_state_indices == nullptr ? b : p.conv_state_indices[b];
+        if (srow < 0) continue;                       // padding slot
+        live[r] = true;
+        sp[r] = reinterpret_cast<u32x4 *>(reinterpret_cast<T *>(p.conv_state) + (int64_t)srow * p.state_stride_b +
+                                          (int64_t)c0 * S);
+        raw[r] = ld_state(sp[r]);
+        const T *xrow = reinterpret_cast<const T *>(p.x) + (int64_t)b * p.x_stride_b + c0;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) xe[r][j] = xrow[j];
+    }
+    // PACKED16: taps and bias packed (dim, W) / (dim,) in the tensors' own 16-bit type, as an inference
+    // checkpoint holds them: whole words of them per lane instead of one 2-byte load per tap.
+    float wv[CH][W], bv[CH];
+    if constexpr (PACKED16) {
+        PackedTaps<W, CH, DT> taps;
+        taps.request(p.weight, p.bias, c0);
+        taps.finish(p.bias != nullptr, wv, bv);
+    } else {
+        load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, w_contiguous_f32 != 0, c0, wv, bv);
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int b = b0 + r;
+        if (b >= p.batch) continue;
+        T *orow = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b + c0;
+        if (!live[r]) {                               // padding slot: zeros out, state untouched
+#pragma unroll
+            for (int j = 0; j < CH; ++j) orow[j] = T(0.f);
+            continue;
+        }
+        T se[CH * S], ne[CH * S];
+        __builtin_memcpy(se, &raw[r], sizeof raw[r]);
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+#pragma unroll
+            for (int q = 0; q + 1 < S; ++q) ne[j * S + q] = se[j * S + q + 1];
+            ne[j * S + S - 1] = xe[r][j];
+        }
+        u32x4 next;
+        __builtin_memcpy(&next, ne, sizeof next);
+        st_state(sp[r], next);
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            float a = bv[j];
+#pragma unroll
+            for (int k = 0; k < W - 1; ++k) a = fmaf(wv[j][k], E::to_float(se[j * S + S - (W - 1) + k]), a);
+            a = fmaf(wv[j][W - 1], E::to_float(xe[r][j]), a);
+            orow[j] = E::from_float(SILU ? silu<PRECISE>(a) : a);
+        }
+    }
+}
+
+#ifndef CC1D_UPDATE_ROWSTATE_ROWS
+#define CC1D_UPDATE_ROWSTATE_ROWS 2
+#endif
+constexpr int kRowStateRows = CC1D_UPDATE_ROWSTATE_ROWS;   // batch entries per lane
+
 // (rows x dim)-shaped operand usable as 16-byte vectors along dim.
 bool rows_vec_ok(const void *ptr, int dtype, int64_t sb, int64_t sc, int64_t sl, int n_rows) {
     const int v = vec_elems(dtype);
@@ -640,6 +733,44 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         if (mode == 1) launch(std::integral_constant<int, 1>{});
         else if constexpr (DT != CC1D_F32) launch(std::integral_constant<int, 2>{});
         return launch_status();
+    }
+    // conv_state (batch, dim, state_len) with unit stride along state_len and whole states in
+    // 16-byte vectors: the row-state kernel.
+    if (p.seqlen == 1 && !circ && p.state_stride_l == 1 && p.state_stride_c == p.state_len && p.x_stride_c == 1 &&
+        p.out_stride_c == 1 && p.batch <= 65535 * kRowStateRows && p.state_len >= W - 1 &&
+        reinterpret_cast<uintptr_t>(p.conv_state) % 16 == 0 &&
+        (p.state_stride_b * (int64_t)Elem<DT>::kBytes) % 16 == 0) {
+        const int state_bytes = p.state_len * Elem<DT>::kBytes;
+        const int ch = state_bytes > 0 && 16 % state_bytes == 0 ? 16 / state_bytes : 0;
+        if (ch >= 1 && ch <= 4 && p.dim % ch == 0) {
+            const uint32_t n_groups = (uint32_t)(p.dim / ch);
+            const dim3 grid((n_groups + kBlock - 1) / kBlock, (uint32_t)((p.batch + kRowStateRows - 1) / kRowStateRows));
+            const int w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
+            bool launched = true;
+            auto go = [&](auto chc) {
+                constexpr int CHC = decltype(chc)::value;
+                if constexpr (16 / (CHC * Elem<DT>::kBytes) >= W - 1 && 16 % (CHC * Elem<DT>::kBytes) == 0 &&
+                              16 / (CHC * Elem<DT>::kBytes) >= 1) {
+                    constexpr bool kCanPack = DT != CC1D_F32 && CHC % 2 == 0;
+                    if (kCanPack && mode == 2) {
+                        if constexpr (kCanPack) {
+                            if (p.silu) hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, true, true, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                            else hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, false, true, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                        }
+                    } else if (p.silu) {
+                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, true, false, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                    } else {
+                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, false, false, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                    }
+                } else {
+                    launched = false;
+                }
+            };
+            if (ch == 1) go(std::integral_constant<int, 1>{});
+            else if (ch == 2) go(std::integral_constant<int, 2>{});
+            else go(std::integral_constant<int, 4>{});
+            if (launched) return launch_status();
+        }
     }
     if (vec) {
         const uint32_t ncg = (uint32_t)(p.dim / Elem<DT>::kVec);

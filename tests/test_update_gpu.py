@@ -100,6 +100,45 @@ def test_update_other_layouts_take_the_element_kernel(pkg, gpu_device, dtype, ci
     assert_close(got, ref, dtype, "out")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width,state_len", [(4, 4), (4, 8), (3, 4), (3, 2), (2, 2), (2, 4), (2, 1), (4, 3), (3, 8)])
+@pytest.mark.parametrize("indices", [False, True])
+def test_update_contiguous_state_rows(pkg, gpu_device, width, state_len, dtype, indices):
+    """conv_state (batch, dim, state_len) contiguous with state_len = d_conv, as mamba_ssm's Mamba
+    block allocates it (unit stride along state_len): whole states in 16-byte vectors take the
+    row-state kernel, the rest (state rows of 6 or 12 bytes, an odd channel count, 16 states of
+    16-bit data) the element kernel; x as (batch, dim) and as (batch, dim, 1)."""
+    g = gen(width * 100 + state_len)
+    dev = gpu_device
+    for dim, batch, two_d in ((2048, 33, True), (5120, 7, False), (1026, 5, True), (517, 3, False)):
+        entries = batch + 9 if indices else batch
+        x = torch.randn(batch, dim, generator=g).to(dtype)
+        if not two_d:
+            x = x.unsqueeze(-1)
+        st = torch.randn(entries, dim, state_len, generator=g).to(dtype)
+        w, b = make_wb(dim, width, True, g)
+        idx = None
+        if indices:
+            idx = torch.randperm(entries, generator=g)[:batch].to(torch.int32)
+            idx[1] = -1
+        st_ref = st.clone()
+        ref = orc.update(x, st_ref, w, b, activation="silu", conv_state_indices=idx)
+        st_dev = st.to(dev)
+        got = pkg.causal_conv1d_update(x.to(dev), st_dev, w.to(dev), b.to(dev), activation="silu",
+                                       conv_state_indices=None if idx is None else idx.to(dev))
+        assert got.shape == x.shape
+        assert torch.equal(st_dev.cpu(), st_ref), (dim, batch)
+        assert_close(got, ref, dtype, "out dim %d" % dim)
+        # taps in the tensors' own 16-bit type, as an inference checkpoint holds them
+        if dtype != torch.float32:
+            st_ref2, st_dev2 = st.clone(), st.to(dev)
+            ref2 = orc.update(x, st_ref2, w.to(dtype).float(), b.to(dtype).float(), activation="silu", conv_state_indices=idx)
+            got2 = pkg.causal_conv1d_update(x.to(dev), st_dev2, w.to(dtype).to(dev), b.to(dtype).to(dev), activation="silu",
+                                            conv_state_indices=None if idx is None else idx.to(dev))
+            assert torch.equal(st_dev2.cpu(), st_ref2)
+            assert_close(got2, ref2, dtype, "out, 16-bit taps, dim %d" % dim)
+
+
 def test_update_golden_and_decode_loop(pkg, gpu_device):
     d = gpu_device
     for case in ("update_linear", "update_circular"):
