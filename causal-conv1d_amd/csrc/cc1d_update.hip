@@ -555,97 +555,135 @@ update_generic_kernel(const cc1d_update_params p, const uint32_t total) {
 }
 
 // Decode step, one token, for conv_state with unit stride along state_len: the (batch, dim,
-// state_len) contiguous cache that mamba_ssm's Mamba block allocates (state_len = d_conv), where a
-// channel's whole state is state_len consecutive elements.  A lane moves one 16-byte vector of
-// it: CH = 16 / (state_len * element size) adjacent channels (two channels of four bf16 states,
-// one of four fp32 states ...), loaded once, shifted by one position in registers
-// (new_state = concat(state, x)[-state_len:], csrc/causal_conv1d_update.cu:72-84,95-98) and stored
-// once; x, out and the taps of those channels are the lane's other accesses, and the taps serve R
-// batch entries.  Grid: x = groups of CH channels / 256, y = batch / R (no division per lane).  Same arithmetic, in the same order,
-// as the other update kernels; the state moves as raw bits.  (256, 5120) bf16, state_len 4, on the same
-// buffers every call / on 40 sets of buffers in turn: 12.4 / 14.6 us with one element access per
-// state position, 4.7 / 6.0-6.3 us here with R = 2 (5.1 / 7.6-7.8 with R = 1, 4.8 / 7.1 with R = 4),
-// 4.7 / 6.1 us for the cache with unit stride along dim.
-template <int DT, int W, int CH, bool SILU, bool PACKED16, int R>
+// state_len) contiguous cache that mamba_ssm's Mamba block allocates (state_len = d_conv) and the
+// (slots, dim, width - 1) cache of paged servers, where a channel's whole state is state_len
+// consecutive elements.  A lane owns CH adjacent channels, the fewest whose states fill whole
+// accesses of VB bytes (two channels of four bf16 states: one 16-byte vector; two channels of three
+// bf16 states: three words ...): it loads them once, shifts every state by one position in
+// registers (new_state = concat(state, x)[-state_len:], csrc/causal_conv1d_update.cu:72-84,95-98)
+// and stores them once; x and out of those channels are one access each.  A workgroup takes 64
+// adjacent channel groups (one per lane) of 4 batch entries (one per wavefront): grid x = channel
+// groups / 64, y = batch / 4, and its taps are fetched once where their layout allows it.  Same
+// arithmetic, in the same order, as the other update kernels; the state moves as raw bits.
+// (256, 5120) bf16, on the same buffers every call / on 40 sets of buffers in turn: state_len 4
+// 4.1-4.4 / 6.1-6.3 us (12.4 / 14.6 us with one element access per state position; 4.7 / 6.1 us for
+// the cache with unit stride along dim), state_len 3 4.5-4.7 / 5.8-5.9 us (4.3 / 5.5), state_len 8
+// 6.1-6.5 / 9.6-9.7 us (7.0 / 13.3).  Two batch entries per lane measured the same or slower.
+// TAPS: how a lane gets its taps.  1 / 2: packed fp32 / packed in the tensors' own 16-bit type and
+// staged once per workgroup through WorkgroupTaps (CH must give whole 8-byte units); 3: packed
+// 16-bit, read per lane in whole words; 0: any layout and type, per lane.
+// Bytes per access to the state: 16 where a state divides 16 bytes or is a multiple of them; 4 for
+// the others (states of 6 or 12 bytes: three elements), where more and narrower lanes measured
+// faster: (256, 5120), state_len 3, 16- / 8- / 4-byte accesses: bf16 6.2 / 5.1 / 4.7 us, fp32 9.0 / 8.5 / 7.3 us.
+#ifndef CC1D_RS_VB
+#define CC1D_RS_VB(state_bytes) ((16 % (state_bytes) == 0 || (state_bytes) % 16 == 0) ? 16 : 4)
+#endif
+template <bool ON, int W, int CH, int WDT> struct RowStateTaps { using type = PackedTaps<W, CH, WDT>; };
+template <int W, int CH, int WDT> struct RowStateTaps<false, W, CH, WDT> { struct type {}; };
+template <bool ON, class Taps, int CH, int W> struct RowStateStaging { using type = WorkgroupTaps<Taps, CH, W>; };
+template <class Taps, int CH, int W> struct RowStateStaging<false, Taps, CH, W> {
+    struct type { static constexpr int kUnits = 1; };
+};
+
+template <int DT, int W, int S, int CH, int VB, int TAPS>
 __global__ void __launch_bounds__(kBlock)
 update_rowstate_kernel(const cc1d_update_params p, const uint32_t n_groups, const int w_contiguous_f32) {
     using E = Elem<DT>;
     using T = typename E::type;
+    using vec_t = typename RawBytes<VB>::type;        // one access to the state
     constexpr bool PRECISE = E::kPreciseAct;
-    constexpr int S = 16 / (CH * E::kBytes);          // state_len
-    static_assert(S * CH * E::kBytes == 16 && S >= W - 1, "one 16-byte vector holds CH whole states");
+    constexpr int NV = CH * S * E::kBytes / VB;       // vectors of state per lane
+    constexpr int XB = CH * E::kBytes;                // bytes of x (and of out) per lane
+    static_assert(NV * VB == CH * S * E::kBytes && S >= W - 1, "CH whole states fill whole vectors");
+    constexpr bool STAGED = TAPS == 1 || TAPS == 2;
+    using Taps = typename RowStateTaps<TAPS != 0, W, CH, (TAPS == 1 ? CC1D_F32 : DT)>::type;
+    using Staging = typename RowStateStaging<STAGED, Taps, CH, W>::type;
+    __shared__ u32x2 staged[Staging::kUnits][kTapRow];
 
-    const uint32_t cg = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
-    if (cg >= n_groups) return;
-    const int c0 = (int)cg * CH;
-    const int b0 = (int)blockIdx.y * R;               // the lane's R batch entries share its taps
+    const uint32_t lc = threadIdx.x & (kWave - 1);
+    const uint32_t col0 = blockIdx.x * (uint32_t)kWave;            // < n_groups by the grid's size
+    const uint32_t cols_here = n_groups - col0 < (uint32_t)kWave ? n_groups - col0 : (uint32_t)kWave;
+    // Lanes past the last channel group shadow the block's first one: every address they form is
+    // valid, and they store nothing.
+    const bool col_ok = lc < cols_here;
+    const int c0 = (int)(col0 + (col_ok ? lc : 0u)) * CH;
+    const int b = (int)blockIdx.y * kStepWaves + __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const bool silu_on = p.silu != 0;
 
-    u32x4 *sp[R];
-    u32x4 raw[R];
-    T xe[R][CH];
-    bool live[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int b = b0 + r;
-        live[r] = false;
-        if (b >= p.batch) continue;
-        const int srow = p.conv_state_indices == nullptr ? b : p.conv_state_indices[b];
-        if (srow < 0) continue;                       // padding slot
-        live[r] = true;
-        sp[r] = reinterpret_cast<u32x4 *>(reinterpret_cast<T *>(p.conv_state) + (int64_t)srow * p.state_stride_b +
+    Staging staging;
+    Taps taps;
+    if constexpr (STAGED) staging.request(p.weight, p.bias, col0, cols_here);
+    if constexpr (TAPS == 3) taps.request(p.weight, p.bias, c0);
+
+    // Wavefronts past the last batch entry and those of a padding slot load nothing.
+    int srow = -1;
+    if (b < p.batch) srow = p.conv_state_indices == nullptr ? b : p.conv_state_indices[b];
+    const bool live = srow >= 0;
+    vec_t *sp = reinterpret_cast<vec_t *>(reinterpret_cast<T *>(p.conv_state) + (int64_t)(live ? srow : 0) * p.state_stride_b +
                                           (int64_t)c0 * S);
-        raw[r] = ld_state(sp[r]);
-        const T *xrow = reinterpret_cast<const T *>(p.x) + (int64_t)b * p.x_stride_b + c0;
+    vec_t raw[NV];
+    T xe[CH];
+    if (live) {
 #pragma unroll
-        for (int j = 0; j < CH; ++j) xe[r][j] = xrow[j];
+        for (int v = 0; v < NV; ++v) raw[v] = ld_state(sp + v);
+        const T *xrow = reinterpret_cast<const T *>(p.x) + (int64_t)b * p.x_stride_b + c0;
+        if constexpr (XB >= 4) {                      // one access: the host checked its alignment
+            using raw_t = typename RawBytes<XB>::type;
+            const raw_t xr = *reinterpret_cast<const raw_t *>(xrow);
+            __builtin_memcpy(xe, &xr, sizeof xr);
+        } else {
+            xe[0] = xrow[0];
+        }
     }
-    // PACKED16: taps and bias packed (dim, W) / (dim,) in the tensors' own 16-bit type, as an inference
-    // checkpoint holds them: whole words of them per lane instead of one 2-byte load per tap.
     float wv[CH][W], bv[CH];
-    if constexpr (PACKED16) {
-        PackedTaps<W, CH, DT> taps;
-        taps.request(p.weight, p.bias, c0);
+    if constexpr (STAGED) {
+        staging.publish(staged);
+        __syncthreads();
+        Staging::collect(staged, lc, taps);
+    }
+    if constexpr (TAPS != 0) {
         taps.finish(p.bias != nullptr, wv, bv);
     } else {
         load_weights<W, CH>(p.weight, p.bias, p.w_dtype, p.w_stride_c, p.w_stride_w, w_contiguous_f32 != 0, c0, wv, bv);
     }
+    if (!col_ok || b >= p.batch) return;
 
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int b = b0 + r;
-        if (b >= p.batch) continue;
-        T *orow = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b + c0;
-        if (!live[r]) {                               // padding slot: zeros out, state untouched
-#pragma unroll
-            for (int j = 0; j < CH; ++j) orow[j] = T(0.f);
-            continue;
-        }
+    T oe[CH];
+    if (live) {
         T se[CH * S], ne[CH * S];
-        __builtin_memcpy(se, &raw[r], sizeof raw[r]);
+        __builtin_memcpy(se, raw, sizeof raw);
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
 #pragma unroll
             for (int q = 0; q + 1 < S; ++q) ne[j * S + q] = se[j * S + q + 1];
-            ne[j * S + S - 1] = xe[r][j];
+            ne[j * S + S - 1] = xe[j];
         }
-        u32x4 next;
-        __builtin_memcpy(&next, ne, sizeof next);
-        st_state(sp[r], next);
+        vec_t next[NV];
+        __builtin_memcpy(next, ne, sizeof next);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) st_state(sp + v, next[v]);
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
             float a = bv[j];
 #pragma unroll
             for (int k = 0; k < W - 1; ++k) a = fmaf(wv[j][k], E::to_float(se[j * S + S - (W - 1) + k]), a);
-            a = fmaf(wv[j][W - 1], E::to_float(xe[r][j]), a);
-            orow[j] = E::from_float(SILU ? silu<PRECISE>(a) : a);
+            a = fmaf(wv[j][W - 1], E::to_float(xe[j]), a);
+            oe[j] = E::from_float(silu_on ? silu<PRECISE>(a) : a);
         }
+    } else {                                          // padding slot: zeros out, state untouched
+#pragma unroll
+        for (int j = 0; j < CH; ++j) oe[j] = T(0.f);
+    }
+    T *orow = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b + c0;
+    if constexpr (XB >= 4) {
+        using raw_t = typename RawBytes<XB>::type;
+        raw_t o;
+        __builtin_memcpy(&o, oe, sizeof o);
+        *reinterpret_cast<raw_t *>(orow) = o;
+    } else {
+        orow[0] = oe[0];
     }
 }
-
-#ifndef CC1D_UPDATE_ROWSTATE_ROWS
-#define CC1D_UPDATE_ROWSTATE_ROWS 2
-#endif
-constexpr int kRowStateRows = CC1D_UPDATE_ROWSTATE_ROWS;   // batch entries per lane
 
 // (rows x dim)-shaped operand usable as 16-byte vectors along dim.
 bool rows_vec_ok(const void *ptr, int dtype, int64_t sb, int64_t sc, int64_t sl, int n_rows) {
@@ -734,43 +772,56 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         else if constexpr (DT != CC1D_F32) launch(std::integral_constant<int, 2>{});
         return launch_status();
     }
-    // conv_state (batch, dim, state_len) with unit stride along state_len and whole states in
-    // 16-byte vectors: the row-state kernel.
+    // conv_state (batch, dim, state_len) with unit stride along state_len: the row-state kernel, for the
+    // state lengths in use (2, 3, 4, 8) when dim is a whole number of lanes' channel groups and a
+    // lane's accesses to the state, x and out are aligned.
     if (p.seqlen == 1 && !circ && p.state_stride_l == 1 && p.state_stride_c == p.state_len && p.x_stride_c == 1 &&
-        p.out_stride_c == 1 && p.batch <= 65535 * kRowStateRows && p.state_len >= W - 1 &&
-        reinterpret_cast<uintptr_t>(p.conv_state) % 16 == 0 &&
-        (p.state_stride_b * (int64_t)Elem<DT>::kBytes) % 16 == 0) {
-        const int state_bytes = p.state_len * Elem<DT>::kBytes;
-        const int ch = state_bytes > 0 && 16 % state_bytes == 0 ? 16 / state_bytes : 0;
-        if (ch >= 1 && ch <= 4 && p.dim % ch == 0) {
-            const uint32_t n_groups = (uint32_t)(p.dim / ch);
-            const dim3 grid((n_groups + kBlock - 1) / kBlock, (uint32_t)((p.batch + kRowStateRows - 1) / kRowStateRows));
-            const int w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
-            bool launched = true;
-            auto go = [&](auto chc) {
-                constexpr int CHC = decltype(chc)::value;
-                if constexpr (16 / (CHC * Elem<DT>::kBytes) >= W - 1 && 16 % (CHC * Elem<DT>::kBytes) == 0 &&
-                              16 / (CHC * Elem<DT>::kBytes) >= 1) {
-                    constexpr bool kCanPack = DT != CC1D_F32 && CHC % 2 == 0;
-                    if (kCanPack && mode == 2) {
-                        if constexpr (kCanPack) {
-                            if (p.silu) hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, true, true, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
-                            else hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, false, true, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
-                        }
-                    } else if (p.silu) {
-                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, true, false, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
-                    } else {
-                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, CHC, false, false, kRowStateRows>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
-                    }
+        p.out_stride_c == 1 && p.state_len >= W - 1 && p.batch <= 65535 * kStepWaves) {
+        bool launched = false;
+        auto run = [&](auto sc) {
+            constexpr int SC = decltype(sc)::value;
+            if constexpr (SC >= W - 1) {
+                constexpr int kStateBytes = SC * Elem<DT>::kBytes;
+                // A lane takes the fewest channels whose states fill whole accesses of VB bytes:
+                // VB / gcd(VB, state bytes).
+                constexpr int VB = CC1D_RS_VB(kStateBytes);
+                constexpr int kGcd = kStateBytes % VB == 0 ? VB : kStateBytes % 8 == 0 && VB >= 8 ? 8 : kStateBytes % 4 == 0 ? 4 : 2;
+                constexpr int CHC = VB / kGcd;
+                constexpr int kLaneBytes = CHC * Elem<DT>::kBytes;
+                if (p.dim % CHC != 0 || reinterpret_cast<uintptr_t>(p.conv_state) % VB != 0 ||
+                    (p.state_stride_b * (int64_t)Elem<DT>::kBytes) % VB != 0) return;
+                if (kLaneBytes >= 4 &&
+                    (!rows_lane_ok(p.x, DT, kLaneBytes, p.x_stride_b, 1, 0, 1) ||
+                     !rows_lane_ok(p.out, DT, kLaneBytes, p.out_stride_b, 1, 0, 1))) return;
+                const uint32_t n_groups = (uint32_t)(p.dim / CHC);
+                const dim3 grid((n_groups + kWave - 1) / kWave, (uint32_t)((p.batch + kStepWaves - 1) / kStepWaves));
+                const int w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
+                constexpr bool kStage32 = CHC % 2 == 0;
+                constexpr bool kStage16 = DT != CC1D_F32 && CHC % 4 == 0;
+                constexpr bool kLane16 = DT != CC1D_F32 && CHC % 2 == 0 && !kStage16;
+                if (mode == 1 && kStage32) {
+                    if constexpr (kStage32)
+                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 1>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                } else if (mode == 2 && kStage16) {
+                    if constexpr (kStage16)
+                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 2>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                } else if (mode == 2 && kLane16) {
+                    if constexpr (kLane16)
+                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 3>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
                 } else {
-                    launched = false;
+                    hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 0>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
                 }
-            };
-            if (ch == 1) go(std::integral_constant<int, 1>{});
-            else if (ch == 2) go(std::integral_constant<int, 2>{});
-            else go(std::integral_constant<int, 4>{});
-            if (launched) return launch_status();
+                launched = true;
+            }
+        };
+        switch (p.state_len) {
+            case 2: run(std::integral_constant<int, 2>{}); break;
+            case 3: run(std::integral_constant<int, 3>{}); break;
+            case 4: run(std::integral_constant<int, 4>{}); break;
+            case 8: run(std::integral_constant<int, 8>{}); break;
+            default: break;
         }
+        if (launched) return launch_status();
     }
     if (vec) {
         const uint32_t ncg = (uint32_t)(p.dim / Elem<DT>::kVec);

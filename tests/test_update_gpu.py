@@ -101,20 +101,23 @@ def test_update_other_layouts_take_the_element_kernel(pkg, gpu_device, dtype, ci
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,state_len", [(4, 4), (4, 8), (3, 4), (3, 2), (2, 2), (2, 4), (2, 1), (4, 3), (3, 8)])
+@pytest.mark.parametrize("width,state_len", [(4, 4), (4, 8), (3, 4), (3, 2), (2, 2), (2, 4), (2, 1), (4, 3), (3, 8),
+                                             (3, 3), (2, 3), (2, 8), (4, 5), (4, 16)])
 @pytest.mark.parametrize("indices", [False, True])
 def test_update_contiguous_state_rows(pkg, gpu_device, width, state_len, dtype, indices):
-    """conv_state (batch, dim, state_len) contiguous with state_len = d_conv, as mamba_ssm's Mamba
-    block allocates it (unit stride along state_len): whole states in 16-byte vectors take the
-    row-state kernel, the rest (state rows of 6 or 12 bytes, an odd channel count, 16 states of
-    16-bit data) the element kernel; x as (batch, dim) and as (batch, dim, 1)."""
+    """conv_state (batch, dim, state_len) contiguous (unit stride along state_len), as mamba_ssm's
+    Mamba block allocates it with state_len = d_conv and paged servers with state_len = width - 1:
+    state lengths 2, 3, 4, 8 take the row-state kernel when dim is a whole number of the lanes'
+    channel groups and x is aligned to a lane's access, the rest (other lengths, an odd channel
+    count, x starting one element off) the element kernel; x as (batch, dim) and as (batch, dim, 1)."""
     g = gen(width * 100 + state_len)
     dev = gpu_device
-    for dim, batch, two_d in ((2048, 33, True), (5120, 7, False), (1026, 5, True), (517, 3, False)):
+    for dim, batch, two_d, x_off in ((2048, 33, True, 0), (5120, 7, False, 0), (1026, 5, True, 0), (517, 3, False, 0),
+                                     (1024, 6, True, 1), (768, 4, True, 2)):
         entries = batch + 9 if indices else batch
-        x = torch.randn(batch, dim, generator=g).to(dtype)
-        if not two_d:
-            x = x.unsqueeze(-1)
+        x_full = torch.randn(batch, dim + 8, generator=g).to(dtype)
+        on_dev = lambda: x_full.to(dev)[:, x_off:x_off + dim] if two_d else x_full.to(dev)[:, :dim].contiguous().unsqueeze(-1)
+        x = x_full[:, x_off:x_off + dim] if two_d else x_full[:, :dim].contiguous().unsqueeze(-1)
         st = torch.randn(entries, dim, state_len, generator=g).to(dtype)
         w, b = make_wb(dim, width, True, g)
         idx = None
@@ -124,7 +127,7 @@ def test_update_contiguous_state_rows(pkg, gpu_device, width, state_len, dtype, 
         st_ref = st.clone()
         ref = orc.update(x, st_ref, w, b, activation="silu", conv_state_indices=idx)
         st_dev = st.to(dev)
-        got = pkg.causal_conv1d_update(x.to(dev), st_dev, w.to(dev), b.to(dev), activation="silu",
+        got = pkg.causal_conv1d_update(on_dev(), st_dev, w.to(dev), b.to(dev), activation="silu",
                                        conv_state_indices=None if idx is None else idx.to(dev))
         assert got.shape == x.shape
         assert torch.equal(st_dev.cpu(), st_ref), (dim, batch)
@@ -133,10 +136,17 @@ def test_update_contiguous_state_rows(pkg, gpu_device, width, state_len, dtype, 
         if dtype != torch.float32:
             st_ref2, st_dev2 = st.clone(), st.to(dev)
             ref2 = orc.update(x, st_ref2, w.to(dtype).float(), b.to(dtype).float(), activation="silu", conv_state_indices=idx)
-            got2 = pkg.causal_conv1d_update(x.to(dev), st_dev2, w.to(dtype).to(dev), b.to(dtype).to(dev), activation="silu",
+            got2 = pkg.causal_conv1d_update(on_dev(), st_dev2, w.to(dtype).to(dev), b.to(dtype).to(dev), activation="silu",
                                             conv_state_indices=None if idx is None else idx.to(dev))
             assert torch.equal(st_dev2.cpu(), st_ref2)
             assert_close(got2, ref2, dtype, "out, 16-bit taps, dim %d" % dim)
+        # no activation, no bias
+        st_ref3, st_dev3 = st.clone(), st.to(dev)
+        ref3 = orc.update(x, st_ref3, w, None, activation=None, conv_state_indices=idx)
+        got3 = pkg.causal_conv1d_update(on_dev(), st_dev3, w.to(dev), None, activation=None,
+                                        conv_state_indices=None if idx is None else idx.to(dev))
+        assert torch.equal(st_dev3.cpu(), st_ref3)
+        assert_close(got3, ref3, dtype, "out, plain, dim %d" % dim)
 
 
 def test_update_golden_and_decode_loop(pkg, gpu_device):
