@@ -2,7 +2,7 @@
 """Benchmark of the causal conv1d hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu] [--no-rotated]
-                    [--no-sustained] [--only update]
+                    [--no-sustained] [--only update] [--decode-calls N]
 
 Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill shape
 (bf16, batch 8, dim 5376, seqlen 2048, channel-last, width 4, bias, SiLU, seq_idx with
@@ -226,7 +226,7 @@ def gbs(n_bytes, us):
 
 
 # ---------------------------------------------------------------------- the other shapes
-def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False):
+def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False, decode_calls=400):
     import torch
     res = {}
 
@@ -246,21 +246,23 @@ def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False):
         n_bytes = update_algorithmic_bytes(cfg, circular)
         out = torch.empty_like(x)
         cs = cfg.get("cache_seqlens")
-        us, wall = time_gpu(lambda i: ext.causal_conv1d_update(x, st, cfg["weight"], cfg["bias"], out, True, cs, None),
-                            steps, warmup)
-        extra = {"us_wall_per_call": round(wall, 2)}
+        # A launch of 4-7 us: a few hundred of them, so that the figure is the device's steady rate
+        # and not the first launches of an empty queue, and no Python work per call beyond the call.
+        n_calls, n_warm = max(steps, decode_calls), max(warmup, decode_calls // 10)
+        update = ext.causal_conv1d_update
+        args = (x, st, cfg["weight"], cfg["bias"], out, True, cs, None)
+        us, wall = time_gpu(lambda i: update(*args), n_calls, n_warm)
+        extra = {"us_wall_per_call": round(wall, 2), "calls_timed": n_calls}
         if rotated:
             sets = clone_sets(cfg, nbytes(x, st, x))
-            outs = [torch.empty_like(s["x"]) for s in sets]
-            def rot(i):
-                s = sets[i % len(sets)]
-                ext.causal_conv1d_update(s["x"], s["conv_state"], s["weight"], s["bias"], outs[i % len(sets)], True,
-                                         s.get("cache_seqlens"), None)
-            us_rot, _ = time_gpu(rot, steps, warmup)
+            rot_args = [(s["x"], s["conv_state"], s["weight"], s["bias"], torch.empty_like(s["x"]), True,
+                         s.get("cache_seqlens"), None) for s in sets]
+            n_sets = len(rot_args)
+            us_rot, _ = time_gpu(lambda i: update(*rot_args[i % n_sets]), n_calls, n_warm)
             extra.update({"us_rotated": round(us_rot, 3), "GBps_rotated": round(gbs(n_bytes, us_rot), 1),
                           "frac_of_hbm_peak_rotated": round(gbs(n_bytes, us_rot) / HBM_PEAK_GBS, 4),
                           "rotated_sets": len(sets)})
-            del sets, outs
+            del sets, rot_args
         # Device duration of the warm launches by rocprofv3 (no dispatch gap in it), from the
         # committed summary of `bench.py --only update`, while the kernel is the one profiled.
         key = "circular_us_device_avg" if circular else "linear_us_device_avg"
@@ -270,6 +272,29 @@ def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False):
     if only_update:
         return res
 
+    # The same step on the cache layout of mamba_ssm's Mamba block and transformers' MambaCache:
+    # conv_state (batch, d_inner, d_conv) contiguous, unit stride along state_len.  Algorithmic
+    # bytes: x, out, taps, bias, the W-1 window positions read and every state position written.
+    cfg = to_dev(config_c3(False, dim=5120), dev)
+    x = cfg["x"]
+    st = torch.randn(x.shape[0], x.shape[1], 4, device=dev).to(x.dtype)
+    out = torch.empty_like(x)
+    n_bytes = nbytes(x, x, cfg["weight"], cfg["bias"]) + nbytes(st) * 7 // 4
+    n_calls, n_warm = max(steps, decode_calls), max(warmup, decode_calls // 10)
+    args = (x, st, cfg["weight"], cfg["bias"], out, True, None, None)
+    us, wall = time_gpu(lambda i: ext.causal_conv1d_update(*args), n_calls, n_warm)
+    extra = {"us_wall_per_call": round(wall, 2), "calls_timed": n_calls,
+             "layout": "conv_state (256, 5120, 4) contiguous, bf16, width 4"}
+    if rotated:
+        n_sets = 40
+        rot_args = [(torch.randn_like(x), torch.randn_like(st), cfg["weight"].clone(), cfg["bias"].clone(),
+                     torch.empty_like(x), True, None, None) for _ in range(n_sets)]
+        us_rot, _ = time_gpu(lambda i: ext.causal_conv1d_update(*rot_args[i % n_sets]), n_calls, n_warm)
+        extra.update({"us_rotated": round(us_rot, 3), "GBps_rotated": round(gbs(n_bytes, us_rot), 1),
+                      "frac_of_hbm_peak_rotated": round(gbs(n_bytes, us_rot) / HBM_PEAK_GBS, 4), "rotated_sets": n_sets})
+        del rot_args
+    record("update_linear_s4_state_contiguous", us, n_bytes, extra)
+
     # What this box charges for any launch of the decode step's size, measured the same way:
     # a device-to-device copy moving as many bytes as the linear step (half read, half written)
     # and a one-element fill (a launch that moves nothing).
@@ -277,8 +302,8 @@ def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False):
     src = torch.empty(half, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
     one = torch.empty(1, device=dev)
-    us_copy, _ = time_gpu(lambda i: dst.copy_(src), 4 * steps, warmup)
-    us_fill, _ = time_gpu(lambda i: one.fill_(1.0), 4 * steps, warmup)
+    us_copy, _ = time_gpu(lambda i: dst.copy_(src), n_calls, n_warm)
+    us_fill, _ = time_gpu(lambda i: one.fill_(1.0), n_calls, n_warm)
     res["launch_floors"] = {"copy_of_update_linear_bytes_us": round(us_copy, 3),
                             "one_element_fill_us": round(us_fill, 3), "copy_bytes": 2 * half}
     del src, dst
@@ -379,6 +404,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-rotated", action="store_true", help="skip the headline over rotating buffer sets")
     ap.add_argument("--no-sustained", action="store_true", help="skip the 400-launch sustained figure")
+    ap.add_argument("--decode-calls", type=int, default=400,
+                    help="launches timed per decode-step figure (at least --steps); counter passes use few")
     ap.add_argument("--only", choices=["update"], default=None,
                     help="time nothing but the warm decode-step launches (linear, then circular): the "
                          "command whose rocprofv3 kernel trace gives their device durations")
@@ -395,7 +422,8 @@ def main():
     import causal_conv1d_cuda as ext          # fails loudly if the extension was not built
     dev = torch.device("cuda:0")
     if args.only == "update":
-        res = bench_others(ext, dev, args.steps, args.warmup, rotated=False, only_update=True)
+        res = bench_others(ext, dev, args.steps, args.warmup, rotated=False, only_update=True,
+                           decode_calls=args.decode_calls)
         print(json.dumps({"only": "update", "steps": args.steps, "warmup": args.warmup, "others": res}), flush=True)
         return
 
@@ -478,7 +506,7 @@ def main():
     del cfg, x, out
     if not args.no_others:
         try:
-            line["others"] = bench_others(ext, dev, args.steps, args.warmup)
+            line["others"] = bench_others(ext, dev, args.steps, args.warmup, decode_calls=args.decode_calls)
         except Exception as e:                                      # keep the headline line intact
             line["others"] = {"error": repr(e)}
     print(json.dumps(line), flush=True)
