@@ -162,6 +162,41 @@ def test_update_state_rows_past_4gib(pkg, gpu_device):
     _free()
 
 
+def test_update_contiguous_state_past_4gib(pkg, gpu_device):
+    """The (slots, dim, state_len) contiguous cache (unit stride along state_len) with slots whose
+    byte offsets do not fit 32 bits, state_len 4 (16-byte accesses) and 3 (word accesses)."""
+    dev, dt = gpu_device, torch.bfloat16
+    D, W, B = 4096, 4, 8
+    for S, N in ((4, 140000), (3, 180000)):              # 2.3e9 and 2.2e9 elements of state
+        state = _randn((N, D, S), dt, dev, 21 + S)
+        assert state.numel() > (1 << 31)
+        idx = torch.tensor([0, N - 1, 131072, 131071, -1, 139000, 65536, 1], dtype=torch.int32, device=dev)
+        rows = idx.clamp(min=0).long()
+        used = idx >= 0
+        w, b = (t.to(dev) for t in make_wb(D, W, True, gen(22)))
+        x = _randn((B, D), dt, dev, 23)
+        small = state[rows].clone()
+        small_idx = torch.arange(B, dtype=torch.int32, device=dev)
+        small_idx[4] = -1
+        untouched = state[N // 2].clone()
+        out = pkg.causal_conv1d_update(x, state, w, b, activation="silu", conv_state_indices=idx)
+        ref = pkg.causal_conv1d_update(x, small, w, b, activation="silu", conv_state_indices=small_idx)
+        assert torch.equal(out, ref)
+        assert not out[4].any()
+        assert torch.equal(state[rows][used], small[used])
+        assert torch.equal(state[N // 2], untouched)
+        # the small call against the oracle: the slots moved as the reference moves them
+        st_cpu = _randn((4, D, S), dt, dev, 31).cpu()
+        st_dev = st_cpu.to(dev)
+        x4 = x[:4].cpu()
+        ref4 = orc.update(x4, st_cpu, w.cpu(), b.cpu(), activation="silu")
+        got4 = pkg.causal_conv1d_update(x4.to(dev), st_dev, w, b, activation="silu")
+        assert torch.equal(st_dev.cpu(), st_cpu)
+        assert_close(got4, ref4, dt, "out")
+        del state
+        _free()
+
+
 def test_varlen_states_tokens_past_4gib(pkg, gpu_device):
     dev, dt = gpu_device, torch.bfloat16
     T, D, S = 1200000, 2048, 3                           # 2.46e9 elements
