@@ -28,12 +28,14 @@ KERNEL_SOURCES = [
     "cc1d_fwd_channellast.hip",
     "cc1d_fwd_channelfirst.hip",
     "cc1d_bwd_channellast.hip",
+    "cc1d_bwd_channellast_lanes4.hip",
+    "cc1d_bwd_channellast_lanes8.hip",
     "cc1d_bwd_channelfirst.hip",
     "cc1d_bwd_noalloc.hip",
     "cc1d_update.hip",
     "cc1d_varlen_states.hip",
 ]
-KERNEL_HEADERS = ["cc1d_device.hpp", "cc1d_internal.hpp"]
+KERNEL_HEADERS = ["cc1d_device.hpp", "cc1d_internal.hpp", "cc1d_bwd_channellast_kernel.hpp"]
 
 LIB_NAME = "libcc1d.so"
 EXT_NAME = "causal_conv1d_cuda" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so")

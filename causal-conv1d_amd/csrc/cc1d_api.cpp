@@ -239,6 +239,7 @@ Knob *find_knob(const char *name) {
         {"fwd_cl_chunk_runs", &Tunables::fwd_cl_chunk_runs},
         {"bwd_cl_rows", &Tunables::bwd_cl_rows},
         {"bwd_cl_chunk_runs", &Tunables::bwd_cl_chunk_runs},
+        {"bwd_cl_lane_bytes", &Tunables::bwd_cl_lane_bytes},
         {"fwd_cf_vecs", &Tunables::fwd_cf_vecs},
         {"bwd_cf_parts", &Tunables::bwd_cf_parts},
         {"launch_limit_shift", &Tunables::launch_limit_shift},

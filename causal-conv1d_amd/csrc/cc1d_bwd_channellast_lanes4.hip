@@ -1,0 +1,11 @@
+// Channel-last backward on 16-bit data with 2 channels (4 bytes) per lane: the instantiations only.
+#include "cc1d_bwd_channellast_kernel.hpp"
+
+namespace cc1d {
+
+int launch_bwd_channellast_16bit_lanes4(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hipStream_t stream) {
+    if (p.x_dtype == CC1D_F16) return launch_dtype<CC1D_F16, CC1D_BWD_CL_CH16>(p, g, ws, stream);
+    return launch_dtype<CC1D_BF16, CC1D_BWD_CL_CH16>(p, g, ws, stream);
+}
+
+}  // namespace cc1d

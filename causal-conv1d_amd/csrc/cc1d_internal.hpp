@@ -64,8 +64,8 @@ struct Knob {
     void set(int32_t x) { v.store(x, std::memory_order_relaxed); }
 };
 struct Tunables {
-    Knob fwd_cl_rows, fwd_cl_half_vec, fwd_cl_chunk_runs, bwd_cl_rows, bwd_cl_chunk_runs, fwd_cf_vecs,
-        bwd_cf_parts, launch_limit_shift;
+    Knob fwd_cl_rows, fwd_cl_half_vec, fwd_cl_chunk_runs, bwd_cl_rows, bwd_cl_chunk_runs, bwd_cl_lane_bytes,
+        fwd_cf_vecs, bwd_cf_parts, launch_limit_shift;
 };
 Tunables &tunables();
 

@@ -272,6 +272,8 @@ int cc1d_hip_runtime_path(char *path, size_t size);
  *   "bwd_cl_rows"   same for the channel-last backward
  *   "bwd_cl_chunk_runs" the same for the channel-last backward, whose workgroups take 4 runs each:
  *                   n >= 4 = chunks of n / 4 workgroup rows; -1 = one contiguous slice per XCD
+ *   "bwd_cl_lane_bytes" bytes of a row per lane in the channel-last backward on 16-bit data: 4 or 8
+ *                   (0: 8 where the rows of dx do not start on 64-byte boundaries, else 4)
  *   "fwd_cf_vecs"   16-byte vectors per wave segment in the channel-first forward
  *   "bwd_cf_parts"  partitions of (batch x seqlen) per channel in the channel-first backward
  *   "launch_limit_shift" n: one launch holds at most 2^(31-n) threads instead of 2^31 (n <= 24), so

@@ -219,6 +219,85 @@ def test_bwd_workgroup_order_does_not_change_results(pkg, gpu_device, cc1d_lib, 
     check(tuple(outs[0]) + (None,), orc.bwd(x, w, b, dout, activation="silu"), dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dim,seqlen,width,has_bias,silu,extras", [
+    (64, 8, 2, True, True, "seq"), (64, 151, 4, True, False, "states"), (72, 372, 3, False, True, "seq"),
+    (4128, 32, 4, True, True, ""), (4128, 784, 4, True, True, "seq"), (1160, 1237, 3, True, True, "states"),
+    (520, 2050, 4, False, False, ""),
+])
+def test_bwd_channel_last_lane_widths_agree(pkg, gpu_device, cc1d_lib, dim, seqlen, width, has_bias, silu, extras, dtype):
+    """Channel-last backward on 16-bit data with 4-byte and with 8-byte lanes (the library takes
+    the wider ones by itself where the rows of dx do not start on 64-byte boundaries): both match
+    the oracle, and dx, a sum per element in one order, is the same bit for bit."""
+    lib = cabi.declare(cc1d_lib)
+    g = gen(dim + seqlen + width)
+    x = make_x(3, dim, seqlen, dtype, True, g)
+    dout = make_x(3, dim, seqlen, dtype, True, g, sliced=False)
+    w, b = make_wb(dim, width, has_bias, g)
+    seq = random_seq_idx(3, seqlen, g) if extras == "seq" else None
+    init = make_states(3, dim, width - 1, dtype, g) if extras == "states" else None
+    dfin = make_states(3, dim, width - 1, dtype, g) if extras == "states" else None
+    act = "silu" if silu else None
+    ref = orc.bwd(x, w, b, dout, seq_idx=seq, initial_states=init, dfinal_states=dfin, activation=act)
+    outs = []
+    try:
+        for lane_bytes in (4, 8):
+            assert lib.cc1d_set_tunable(b"bwd_cl_lane_bytes", lane_bytes) == 0
+            outs.append(run_gpu(pkg, gpu_device, x, w, b, dout, seq=seq, init=init, dfin=dfin, act=act))
+    finally:
+        lib.cc1d_set_tunable(b"bwd_cl_lane_bytes", 0)
+    for got in outs:
+        check(got, ref, dtype)
+    assert torch.equal(outs[0][0], outs[1][0])
+    if outs[0][3] is not None:
+        assert torch.equal(outs[0][3], outs[1][3])
+
+
+def test_bwd_dx_as_column_slice_of_a_wider_tensor(gpu_device, cc1d_lib):
+    """The layout of mamba_ssm's Mamba-2 backward: x and dx are column slices of tensors d_in_proj
+    wide (rows that do not start on 64-byte boundaries), dout is dense; a launch large enough that
+    the library picks its lane width from the alignment of dx.  Against the oracle on one batch
+    entry and, bit for bit, against the same call with dense tensors."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    B, L, D, d_in_proj, off = 16, 2048, 1792, 3352, 1536
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    big_x = torch.randn(B, L, d_in_proj, generator=g, device=dev).to(torch.bfloat16)
+    big_dx = torch.zeros(B, L, d_in_proj, device=dev, dtype=torch.bfloat16)
+    x = big_x[:, :, off:off + D].transpose(1, 2)
+    dx = big_dx[:, :, off:off + D].transpose(1, 2)
+    dout = torch.randn(B, L, D, generator=g, device=dev).to(torch.bfloat16).transpose(1, 2)
+    w, b = (t.to(dev) for t in make_wb(D, 4, True, gen(6)))
+    seq = torch.zeros(B, L, dtype=torch.int32, device=dev)
+    seq[:, 700:] = 1
+    seq[:, 1500:] = 2
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(xv, dxv):
+        dw = torch.zeros(D, 4, device=dev)
+        db = torch.zeros(D, device=dev)
+        p = cabi.bwd_params(xv, w, b, dout, dxv, dw, db, True, seq_idx=seq)
+        need = ctypes.c_size_t()
+        assert lib.cc1d_bwd_workspace_bytes(ctypes.byref(p), ctypes.byref(need)) == 0
+        ws = torch.empty(max(16, need.value), dtype=torch.uint8, device=dev)
+        st = lib.cc1d_bwd(ctypes.byref(p), ws.data_ptr(), need.value, stream)
+        assert st == 0, lib.cc1d_strerror(st)
+        torch.cuda.synchronize()
+        return dw, db
+
+    dw, db = run(x, dx)
+    assert not big_dx[:, :, :off].any() and not big_dx[:, :, off + D:].any()     # nothing outside the slice
+    dense_x = x.transpose(1, 2).contiguous().transpose(1, 2)
+    dense_dx = torch.empty_like(dense_x)
+    dw2, db2 = run(dense_x, dense_dx)
+    assert torch.equal(dx, dense_dx)
+    assert_close(dw, dw2, what="dweight", tol=TOL_W)
+    assert_close(db, db2, what="dbias", tol=TOL_W)
+    ref = orc.bwd(x[5:6].cpu(), w.cpu(), b.cpu(), dout[5:6].cpu(), seq_idx=seq[5:6].cpu(), activation="silu")
+    assert_close(dx[5:6], ref[0].to(torch.bfloat16), torch.bfloat16, "dx")
+
+
 @pytest.mark.parametrize("channel_last", [False, True])
 def test_bwd_c_abi_accumulates_into_dweight(gpu_device, cc1d_lib, channel_last):
     """Through the C ABI with a caller-owned workspace: dweight / dbias are added to, as the
