@@ -66,3 +66,30 @@ def test_decode_step(pkg, gpu_device, dtype, w_dtype, seqlen, circular, has_bias
                                    cache_seqlens=None if cs is None else cs.to(dev))
     assert torch.equal(st_dev.cpu(), st_ref), "conv_state must be bit-exact"
     assert_close(got, ref.to(dtype), dtype, "out")
+
+
+@pytest.mark.parametrize("width,state_len", [(2, 2), (3, 3), (4, 3), (4, 4), (4, 8)])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("dtype,w_dtype", PAIRS)
+def test_decode_step_contiguous_state(pkg, gpu_device, dtype, w_dtype, has_bias, width, state_len):
+    """conv_state (batch, dim, state_len) contiguous (the row-state kernel): taps of every
+    supported type, packed or as a strided view."""
+    dev = gpu_device
+    g = gen(200 + width + state_len)
+    B, D = 9, 328
+    x = torch.randn(B, D, generator=g).to(dtype)
+    st = torch.randn(B, D, state_len, generator=g).to(dtype)
+    w, b = make_wb(D, width, has_bias, g, w_dtype)
+    for strided in (False, True):
+        wd = w.to(dev)
+        if strided:                                       # a column slice of a wider tensor: the general loader
+            wide = torch.zeros(D, width + 3, dtype=w_dtype, device=dev)
+            wide[:, 1:1 + width] = wd
+            wd = wide[:, 1:1 + width]
+        st_ref = st.clone()
+        ref = orc.update(x, st_ref, w.float(), None if b is None else b.float(), activation="silu")
+        st_dev = st.to(dev)
+        got = pkg.causal_conv1d_update(x.to(dev), st_dev, wd, None if b is None else b.to(dev), activation="silu")
+        assert torch.equal(st_dev.cpu(), st_ref), "conv_state must be bit-exact"
+        assert_close(got, ref.to(dtype), dtype, "out")
+
