@@ -31,6 +31,17 @@
 #include "cc1d_device.hpp"
 #include "cc1d_internal.hpp"
 
+// Rows of more than three steps start their steps on 128-byte lines of out (one more, partly
+// filled step per row); shorter rows start them at the row's first vector.  (8, 5376, L) bf16, steps
+// at the first vector / on lines: L = 1000 32.7 / 38.3 us, 1500 54.7 / 57.3, 2000 62.6 / 57.0, 2400 72.2 / 66.0,
+// 3000 101.7 / 84.3, 4080 151 / 133, 6000 200 / 177; fp32 L = 1000 64.7 / 56.6, 1500 103.3 / 83.8 us.
+#ifndef CC1D_FWD_CF_ALIGN_MIN_VECS
+#define CC1D_FWD_CF_ALIGN_MIN_VECS 193
+#endif
+#ifndef CC1D_FWD_CF_U2_STEPS
+#define CC1D_FWD_CF_U2_STEPS 8
+#endif
+
 namespace cc1d {
 namespace {
 
@@ -39,6 +50,7 @@ struct FwdCfGeom {
     int32_t vecs_per_seg;     // multiple of 64
     int32_t n_segs;           // segments per row
     uint32_t total_waves;     // batch * dim * n_segs
+    int32_t lead_vecs;        // streaming kernel: 7 = a row's steps start on 128-byte lines of out, 0 = at the row's first vector
 };
 
 // Row number of the launch -> (batch entry, channel).  Channels run fastest for tensors whose rows
@@ -216,20 +228,32 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
     const T *xr = reinterpret_cast<const T *>(p.x) + xrow;
     T *orow = reinterpret_cast<T *>(p.out) + (int64_t)b * p.out_stride_b + (int64_t)c * p.out_stride_c;
 
-    // The row on its own 16-byte grid (x and out share it): vector j holds positions
-    // j*VEC - mis .. j*VEC - mis + VEC.  Vectors jf0 .. jf1 lie inside the row and move as
-    // vectors; the up to VEC-1 positions in front of them and behind them are edge positions,
-    // each produced by one lane straight from memory.
-    const int mis = (int)((reinterpret_cast<uintptr_t>(xr) / sizeof(T)) % VEC);
-    const int jf0 = mis > 0 ? 1 : 0;
+    // The row on its own 16-byte grid (x and out share it), with the grid's origin moved back to
+    // the 128-byte line of out that holds the row's first vector: vector j holds positions
+    // j*VEC - mis .. j*VEC - mis + VEC, and a step of 64 vectors starts on a line.  (Steps that
+    // start inside a line share a 64-byte block with the step before and the step after, and
+    // blocks written in two parts are what such rows lose their time on: (8, 5376, 2000) bf16
+    // 75.6 us against 60.7 us at seqlen 2048, (8, 5376, 4080) 167 against 116 us at 4096.)
+    // Vectors jf0 .. jf1 lie inside the row and move as vectors; the up to VEC-1 positions in front
+    // of them and behind them are edge positions, each produced by one lane straight from memory.
+    const int mis0 = (int)((reinterpret_cast<uintptr_t>(xr) / sizeof(T)) % VEC);
+    const int lead = g.lead_vecs == 0 ? 0 : (int)(((reinterpret_cast<uintptr_t>(orow) - (uintptr_t)mis0 * sizeof(T)) / 16) % 8);
+    const int mis = mis0 + lead * VEC;                // elements between the grid's origin and the row start
+    const int jf0 = (mis + VEC - 1) / VEC;            // 0 .. 8
     const int jf1 = (L + mis) / VEC;
-    int j_begin = seg * g.vecs_per_seg;
+    const int j0 = seg * g.vecs_per_seg;              // the segment's steps start here, on a line
+    int j_begin = j0;
     int j_end = j_begin + g.vecs_per_seg;
     const bool owns_tail = j_begin <= jf1 && jf1 < j_end;
     if (j_begin < jf0) j_begin = jf0;
     if (j_end > jf1) j_end = jf1;
+    // A first step whose leading lanes lie in front of the row's first whole vector (the row's
+    // first segment, when the row does not start on a line) is done on its own, checked.
+    const bool head = j_begin > j0 && j_begin < j_end;
+    const int s_first = head ? 1 : 0;
     // whole groups of U steps, in pairs
-    const int n_groups = j_begin < j_end ? (j_end - j_begin) / (2 * kWave * U) * 2 : 0;
+    const int n_full = j_begin < j_end ? (j_end - j0) / kWave - s_first : 0;
+    const int n_groups = n_full > 0 ? n_full / (2 * U) * 2 : 0;
 
     float wv[W], bias_v;
 #pragma unroll
@@ -246,7 +270,7 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
     // of the wave whose range holds vector jf1.  A row shorter than its first vector is all
     // front edge.
     {
-        const int front = mis == 0 ? 0 : (jf1 < jf0 ? L : VEC - mis);
+        const int front = jf1 < jf0 ? L : jf0 * VEC - mis;
         const int back = jf1 < jf0 ? L : jf1 * VEC - mis;
         int t = -1;
         if (seg == 0 && lane < front) t = lane;
@@ -267,8 +291,8 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
         for (int i = 0; i < W - 1; ++i)
             carry[i] = padded_elem<DT, W>(p, xrow, b, c, j_begin * VEC - mis - (W - 1) + i);
 
-        const T *xs = xr - mis + (j_begin + lane) * VEC;    // this lane's vector of step 0
-        T *os = orow - mis + (j_begin + lane) * VEC;
+        const T *xs = xr - mis + (j0 + s_first * kWave + lane) * VEC;    // this lane's vector of the first whole step
+        T *os = orow - mis + (j0 + s_first * kWave + lane) * VEC;
         auto load_group = [&](int k, u32x4 (&raw)[U]) {
 #pragma unroll
             for (int u = 0; u < U; ++u)
@@ -300,54 +324,71 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
             }
         };
 
-        // Two register sets of U steps in ping-pong; the first and last pair of groups are
-        // peeled so the loop is entered in the state its back edge leaves and the wait counts
-        // stay exact.
+        // The checked first step's vector is requested first and the first two groups of whole
+        // steps right behind it, so that its arithmetic runs while they are in flight.
+        const int first = j_begin - j0;               // head: 1 .. 8
+        const bool head_mine = head && lane >= first && j0 + lane < j_end;
+        u32x4 head_raw = u32x4{0u, 0u, 0u, 0u};
+        if (head_mine) head_raw = *reinterpret_cast<const u32x4 *>(xs - kWave * VEC);
+        // Steps the whole pairs do not cover (fewer than 2 U whole ones and possibly a partly filled
+        // one) are two more groups, requested and computed in the same ping-pong with every lane
+        // checked: lanes past the segment's end read zeros and store nothing.  They use the
+        // non-temporal policy of the whole steps: with plain accesses for them, (8, 5376, 2000) bf16
+        // took 65.6 us against 58.3 us, (8, 5376, 3000) 100.0 against 84.5 us and fp32 (8, 5376, 1000)
+        // 66.5 against 56.7 us.  (The checked first step keeps plain accesses: 58.3 against 60.2 us and
+        // 84.5 against 92.2 us.)
+        auto load_group_checked = [&](int k, u32x4 (&raw)[U]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                raw[u] = u32x4{0u, 0u, 0u, 0u};
+                if (j0 + (s_first + k * U + u) * kWave + lane < j_end)
+                    raw[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(xs + (k * U + u) * (kWave * VEC)));
+            }
+        };
+        auto compute_group_checked = [&](int k, const u32x4 (&raw)[U]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (j0 + (s_first + k * U + u) * kWave >= j_end) break;       // wave-uniform
+                const bool mine = j0 + (s_first + k * U + u) * kWave + lane < j_end;
+                float xf[VEC];
+                E::unpack(raw[u], xf);
+                float xx[VEC + W - 1];
+#pragma unroll
+                for (int i = 0; i < W - 1; ++i) {
+                    xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry[i]);
+                    carry[i] = read_lane(xf[VEC - (W - 1) + i], kWave - 1);
+                }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xf[e];
+                float acc[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float a = bias_v;
+#pragma unroll
+                    for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
+                    acc[e] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
+                }
+                if (mine) __builtin_nontemporal_store(E::pack(acc), reinterpret_cast<u32x4 *>(os + (k * U + u) * (kWave * VEC)));
+            }
+        };
         u32x4 ra[U], rb[U];
         if (n_groups >= 2) {
             load_group(0, ra);
             load_group(1, rb);
-            if (n_groups == 2) {
-                compute_group(0, ra);
-                compute_group(1, rb);
-            } else {
-                compute_group(0, ra);
-                load_group(2, ra);
-                compute_group(1, rb);
-                load_group(3, rb);
-                int k = 2;
-#pragma clang loop unroll(disable)
-                for (; k + 2 < n_groups; k += 2) {
-                    compute_group(k, ra);
-                    load_group(k + 2, ra);
-                    compute_group(k + 1, rb);
-                    load_group(k + 3, rb);
-                }
-                compute_group(k, ra);
-                compute_group(k + 1, rb);
-            }
+        } else {
+            load_group_checked(0, ra);
+            load_group_checked(1, rb);
         }
-        // Steps the pairs did not cover (fewer than 2 U whole ones and possibly a partly filled
-        // one): all requested first, lanes past the segment's end read zeros and store nothing.
-        constexpr int kTail = 2 * U;
-        const int s0 = n_groups * U;                  // first step of the tail
-        u32x4 tail[kTail];
-#pragma unroll
-        for (int q = 0; q < kTail; ++q) {
-            tail[q] = u32x4{0u, 0u, 0u, 0u};
-            if (j_begin + (s0 + q) * kWave + lane < j_end)
-                tail[q] = *reinterpret_cast<const u32x4 *>(xs + (s0 + q) * (kWave * VEC));
-        }
-#pragma unroll
-        for (int q = 0; q < kTail; ++q) {
-            if (j_begin + (s0 + q) * kWave >= j_end) break;
-            const bool mine = j_begin + (s0 + q) * kWave + lane < j_end;
+        if (head) {
+            // Lanes in front of the row's first whole vector load and store nothing; the one right
+            // in front of it hands the halo on.
             float xf[VEC];
-            E::unpack(tail[q], xf);
+            E::unpack(head_raw, xf);
             float xx[VEC + W - 1];
 #pragma unroll
             for (int i = 0; i < W - 1; ++i) {
-                xx[i] = from_prev_lane(xf[VEC - (W - 1) + i], carry[i]);
+                const float top = lane == first - 1 ? carry[i] : xf[VEC - (W - 1) + i];
+                xx[i] = from_prev_lane(top, 0.f);
                 carry[i] = read_lane(xf[VEC - (W - 1) + i], kWave - 1);
             }
 #pragma unroll
@@ -360,8 +401,29 @@ fwd_channelfirst_stream_kernel(const cc1d_fwd_params p, const FwdCfGeom g) {
                 for (int w = 0; w < W; ++w) a = fmaf(wv[w], xx[e + w], a);
                 acc[e] = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
             }
-            if (mine) *reinterpret_cast<u32x4 *>(os + (s0 + q) * (kWave * VEC)) = E::pack(acc);
+            if (head_mine) *reinterpret_cast<u32x4 *>(os - kWave * VEC) = E::pack(acc);
         }
+
+        // Two register sets of U steps in ping-pong: while one group is computed and stored the
+        // loads of the next two are in flight.  The whole groups (an even number) come first,
+        // unchecked; the two checked groups close the walk in the same rhythm.
+        int k = 0;
+        if (n_groups >= 2) {
+#pragma clang loop unroll(disable)
+            for (; k + 2 < n_groups; k += 2) {
+                compute_group(k, ra);
+                load_group(k + 2, ra);
+                compute_group(k + 1, rb);
+                load_group(k + 3, rb);
+            }
+            compute_group(k, ra);
+            load_group_checked(k + 2, ra);
+            compute_group(k + 1, rb);
+            load_group_checked(k + 3, rb);
+            k += 2;
+        }
+        compute_group_checked(k, ra);
+        compute_group_checked(k + 1, rb);
     }
 
     // final_states[b, c, i] = xpad[L-(W-1)+i], bit-exact copies, by the row's first wave.
@@ -720,11 +782,17 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     const bool same_grid = (reinterpret_cast<uintptr_t>(p.x) - reinterpret_cast<uintptr_t>(p.out)) % 16 == 0 &&
                            reinterpret_cast<uintptr_t>(p.x) % eb == 0 &&
                            (p.x_stride_b - p.out_stride_b) % vec == 0 && (p.x_stride_c - p.out_stride_c) % vec == 0;
-    const int streaming = !same_grid ? 0 : p.seqlen >= 8 * kWave * vec ? 2 : 1;
+    const int streaming = !same_grid ? 0 : p.seqlen >= CC1D_FWD_CF_U2_STEPS * kWave * vec ? 2 : 1;
     // Vectors a row can span on its grid: exact when every row starts on the grid, else the
     // worst case (a row may start up to vec-1 elements into its first vector).
     const bool on_grid = aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0;
-    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + (on_grid && streaming ? 0 : vec - 1)) / vec;
+    // The streaming kernel moves a row's grid back to the 128-byte line of out its first vector
+    // lies in: up to seven more vectors, unless every row of out starts on a line.
+    const bool rows_on_lines = on_grid && reinterpret_cast<uintptr_t>(p.out) % 128 == 0 &&
+                               (p.out_stride_b * eb) % 128 == 0 && (p.out_stride_c * eb) % 128 == 0;
+    const bool align_steps = streaming && !rows_on_lines && ((int64_t)p.seqlen + vec - 1) / vec >= CC1D_FWD_CF_ALIGN_MIN_VECS;
+    const int64_t lead_max = align_steps ? 7 * vec : 0;
+    const int64_t max_vecs = ((int64_t)p.seqlen + vec - 1 + lead_max + (on_grid && streaming ? 0 : vec - 1)) / vec;
     const int64_t rows = (int64_t)p.batch * p.dim;
     // Short rows of whole vectors, up to eight to a wavefront, no walk: (4, 5376, 256) bf16 11.2 -> 6.0 us,
     // (8, 1024, 512) bf16 6.7 -> 4.8 us, (4, 5376, 256) fp32 10.9 -> 8.5 us, (1, 5376, 64) bf16 4.8 -> 3.3 us.
@@ -777,6 +845,7 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
     if (vps < quantum) vps = quantum;
     FwdCfGeom g;
     g.streaming = streaming;
+    g.lead_vecs = align_steps ? 7 : 0;
     g.vecs_per_seg = (int32_t)vps;
     g.n_segs = (int32_t)((max_vecs + vps - 1) / vps);
     const int64_t total = rows * g.n_segs;

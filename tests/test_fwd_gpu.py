@@ -264,6 +264,39 @@ def test_fwd_launch_geometry_does_not_change_results(pkg, gpu_device, cc1d_lib, 
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seqlen", [1544, 1552, 2000, 2047, 3000, 4104, 9000])
+def test_fwd_channel_first_rows_off_the_cache_lines(pkg, gpu_device, cc1d_lib, seqlen, dtype):
+    """Channel-first rows longer than three steps whose ends do not fall on 128-byte lines: the walk
+    starts its steps on lines of out, with a partly filled first step and, where rows are cut, with
+    segments that start on lines too.  Every segment length gives the same bits; initial and final
+    states; a view whose rows start anywhere on the 16-byte grid."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    g = gen(1000 + seqlen)
+    B, D, W = 2, 24, 4
+    big = torch.randn(B, D, seqlen + 24, generator=g).to(dtype)
+    w, b = make_wb(D, W, True, g)
+    init = make_states(B, D, W - 1, dtype, g)
+    for off in (0, 8, 16 // big.element_size(), 3):
+        x = big[:, :, off:off + seqlen]
+        ref, fin = orc.fwd(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+        xd = big.to(dev)[:, :, off:off + seqlen]
+        outs = []
+        try:
+            for vecs in (0, 128, 256, 1024):
+                assert lib.cc1d_set_tunable(b"fwd_cf_vecs", vecs) == 0
+                o, f = pkg.causal_conv1d_fn(xd, w.to(dev), b.to(dev), initial_states=init.to(dev),
+                                            return_final_states=True, activation="silu")
+                outs.append((o.cpu(), f.cpu()))
+        finally:
+            lib.cc1d_set_tunable(b"fwd_cf_vecs", 0)
+        for o, f in outs[1:]:
+            assert torch.equal(o, outs[0][0]) and torch.equal(f, outs[0][1])
+        assert_close(outs[0][0], ref, dtype, "out, offset %d" % off)
+        assert torch.equal(outs[0][1], fin)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_fwd_workgroup_order_does_not_change_results(pkg, gpu_device, cc1d_lib, dtype):
     """The channel-last forward hands its workgroups to the XCDs in contiguous slices or in chunks
     of runs, by shape; every order covers every run exactly once: same bits, ragged last run and
