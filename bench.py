@@ -269,9 +269,6 @@ def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False, decod
         if key in prof:
             extra.update({"us_device_rocprof": float(prof[key]), "us_device_rocprof_source": prof["profile"]})
         record(name, us, n_bytes, extra)
-    if only_update:
-        return res
-
     # The same step on the cache layout of mamba_ssm's Mamba block and transformers' MambaCache:
     # conv_state (batch, d_inner, d_conv) contiguous, unit stride along state_len.  Algorithmic
     # bytes: x, out, taps, bias, the W-1 window positions read and every state position written.
@@ -293,7 +290,12 @@ def bench_others(ext, dev, steps, warmup, rotated=True, only_update=False, decod
         extra.update({"us_rotated": round(us_rot, 3), "GBps_rotated": round(gbs(n_bytes, us_rot), 1),
                       "frac_of_hbm_peak_rotated": round(gbs(n_bytes, us_rot) / HBM_PEAK_GBS, 4), "rotated_sets": n_sets})
         del rot_args
+    if "contiguous_us_device_avg" in prof:
+        extra.update({"us_device_rocprof": float(prof["contiguous_us_device_avg"]), "us_device_rocprof_source": prof["profile"]})
     record("update_linear_s4_state_contiguous", us, n_bytes, extra)
+
+    if only_update:
+        return res
 
     # What this box charges for any launch of the decode step's size, measured the same way:
     # a device-to-device copy moving as many bytes as the linear step (half read, half written)
