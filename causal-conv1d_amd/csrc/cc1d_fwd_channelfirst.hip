@@ -21,9 +21,10 @@
 // empty_like gives): whole 64-vector steps run without bounds checks in two register sets in
 // ping-pong, which keep the loads of the next two groups in flight while a group is computed
 // and stored; what is left over at the end of a segment (fewer than a pair of groups, a partly
-// filled step) is requested at once and then worked off step by step, and the few positions of
-// a row in front of its first whole vector or behind its last one are produced one per lane,
-// straight from memory.  The general kernel takes out tensors on a different grid.  The short-row
+// filled step) is two more groups in the same ping-pong with every lane checked; rows of more than
+// three steps start their steps on 128-byte lines of out, with a partly filled first step; and
+// the few positions of a row in front of its first whole vector or behind its last one are
+// produced one per lane, straight from memory.  The general kernel takes out tensors on a different grid.  The short-row
 // kernel takes rows of at most 64 vectors, several rows to a wavefront and no walk; the flat
 // kernel takes such rows of a contiguous tensor as whole vectors of one flat array.
 #include <type_traits>
