@@ -2,7 +2,7 @@
 """Benchmark of the causal conv1d hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu] [--no-rotated]
-                    [--no-sustained] [--only update] [--decode-calls N]
+                    [--no-settle] [--only update|rotated] [--decode-calls N]
 
 Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill shape
 (bf16, batch 8, dim 5376, seqlen 2048, channel-last, width 4, bias, SiLU, seq_idx with
@@ -12,12 +12,15 @@ Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill 
                      algorithmic bytes count every input element read once and every
                      output element written once (x, out, seq_idx, weight, bias)
   roofline ......... the same bytes over the average kernel time measured with HIP events
-                     around the timed launches, against the 8 TB/s HBM3E peak.  `frac` is the
-                     warm burst the K timed steps are (one set of buffers, a few milliseconds of
-                     load); `frac_sustained` the same call over 400 back-to-back launches, past
-                     the point where the clock settles; `frac_rotated` over six rotating sets of
-                     x and out (2.1 GB), where every launch meets cold caches and address
-                     translations, as the layers of a model do
+                     around the timed launches, against the 8 TB/s HBM3E peak.  `frac` (and
+                     `value`) is the sustained rate: the K timed steps follow 400 untimed
+                     back-to-back launches of the same call, so the clock has settled where it
+                     stays under load; `frac_burst` is the same K steps out of an idle device
+                     (a few milliseconds of load at the highest clock); `frac_rotated` runs over
+                     six rotating sets of x and out (2.1 GB), where every launch meets cold caches
+                     and address translations, as the layers of a model do.  `decode` repeats
+                     the three figures for the two decode-step updates.  `traffic` is imported
+                     from the committed rocprofv3 summary, not measured in this run
   cpu_baseline ..... the PyTorch oracle (F.conv1d per packed sub-sequence) timed on this
                      host's cores on the same inputs
   others ........... µs per call and GB/s of the remaining shapes: decode-step update
@@ -405,12 +408,15 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="time only the headline forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host CPU baseline")
     ap.add_argument("--no-rotated", action="store_true", help="skip the headline over rotating buffer sets")
-    ap.add_argument("--no-sustained", action="store_true", help="skip the 400-launch sustained figure")
+    ap.add_argument("--no-settle", action="store_true",
+                    help="time the K steps out of an idle device (the burst figure) instead of after 400 "
+                         "untimed launches; `value` is then the burst")
     ap.add_argument("--decode-calls", type=int, default=400,
                     help="launches timed per decode-step figure (at least --steps); counter passes use few")
-    ap.add_argument("--only", choices=["update"], default=None,
-                    help="time nothing but the warm decode-step launches (linear, then circular): the "
-                         "command whose rocprofv3 kernel trace gives their device durations")
+    ap.add_argument("--only", choices=["update", "rotated"], default=None,
+                    help="update: time nothing but the warm decode-step launches (linear, then circular); "
+                         "rotated: nothing but the headline forward over its six rotating buffer sets.  The "
+                         "commands whose rocprofv3 kernel traces and counters give device durations and traffic")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of x (a kernel of known size, to scale profiler counters)")
     args = ap.parse_args()
@@ -438,7 +444,27 @@ def main():
     def step(i):
         ext.causal_conv1d_fwd(x, w, b, seq, None, out, None, True)
 
-    us, wall_us = time_gpu(step, args.steps, args.warmup)
+    def rotated_sets():
+        # Six sets of x and out (2.1 GB): a launch never finds its tensors in a cache.
+        return [(x, out)] + [(torch.randn_like(x), torch.empty_like(x)) for _ in range(5)]
+
+    if args.only == "rotated":
+        sets = rotated_sets()
+        rot_us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(sets[i % 6][0], w, b, seq, None, sets[i % 6][1], None, True),
+                             args.steps, args.warmup)
+        print(json.dumps({"only": "rotated", "steps": args.steps, "warmup": args.warmup, "rotated_sets": 6,
+                          "us_per_call_rotated": round(rot_us, 3), "algorithmic_bytes": int(n_bytes),
+                          "frac_rotated": round(gbs(n_bytes, rot_us) / HBM_PEAK_GBS, 4)}), flush=True)
+        return
+
+    # The burst: K steps out of an idle device.  Then the figure the line carries: the same K steps
+    # right behind 400 untimed launches (about 22 ms of load), where the clock has settled.
+    burst_us, burst_wall = time_gpu(step, args.steps, args.warmup)
+    if args.no_settle:
+        us, wall_us, settle = burst_us, burst_wall, 0
+    else:
+        settle = 400
+        us, wall_us = time_gpu(step, args.steps, args.warmup + settle)
     if args.copy_probe:
         flat_src = torch.empty(x.numel(), dtype=x.dtype, device=dev).normal_()
         flat_dst = torch.empty_like(flat_src)
@@ -471,30 +497,27 @@ def main():
         "config": {"workload": "Mamba-2 2.7B prefill forward: bf16 x (8, 5376, 2048) channel-last, width 4, "
                                "bias, SiLU, int32 seq_idx with 1-4 packed sub-sequences per row",
                    "algorithmic_bytes": int(n_bytes), "us_per_call": round(us, 3),
+                   "timed": "K steps behind %d untimed back-to-back launches (sustained clock)" % settle
+                            if settle else "K steps out of an idle device (burst)",
+                   "us_per_call_burst": round(burst_us, 3),
                    "us_per_call_python_api_wall": round(api_wall, 2)},
         "roofline": {"bound": "hbm", "achieved": round(gbs(n_bytes, us), 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs(n_bytes, us) / HBM_PEAK_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(gbs(n_bytes, us) / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac_burst": round(gbs(n_bytes, burst_us) / HBM_PEAK_GBS, 4)},
     }
     # HBM bytes per launch by FETCH_SIZE / WRITE_SIZE: only rocprofv3 can read those, so the figure
-    # comes from the committed summary, and only while the kernel sources are the ones it was
+    # is imported from the committed summary, and only while the kernel sources are the ones it was
     # read on (the summary names them by hash); otherwise null.
     prof = profile_figures("fwd_channellast_prefill_traffic.txt", FWD_CL_SOURCES)
     if "traffic_bytes_per_launch" in prof:
         line["roofline"]["traffic"] = int(float(prof["traffic_bytes_per_launch"]))
-        line["roofline"]["traffic_source"] = {"profile": prof["profile"],
+        line["roofline"]["traffic_source"] = {"profile": prof["profile"], "imported": True,
                                               "kernel_sources_sha16": prof["kernel_sources_sha16"]}
-    if not args.no_sustained:
-        # The same call 400 times back to back (about 25 ms of load): the clock settles after the
-        # first few milliseconds, which the K timed steps above mostly end before.
-        sus_us, _ = time_gpu(step, 400, 0)
-        line["config"]["us_per_call_sustained"] = round(sus_us, 3)
-        line["config"]["sustained_steps"] = 400
-        line["roofline"]["frac_sustained"] = round(gbs(n_bytes, sus_us) / HBM_PEAK_GBS, 4)
     if not args.no_others and not args.no_rotated:
         # The same call over six rotating sets of x and out (2.1 GB): every launch then meets cold
         # address translations and caches, as the layers of a model do; next to it PyTorch's
         # elementwise add over the same sets (the same bytes in, the same bytes out).
-        sets = [(x, out)] + [(torch.randn_like(x), torch.empty_like(x)) for _ in range(5)]
+        sets = rotated_sets()
         rot_us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(sets[i % 6][0], w, b, seq, None, sets[i % 6][1], None, True),
                              args.steps, args.warmup)
         add_us, _ = time_gpu(lambda i: torch.add(sets[i % 6][0], 1.0, out=sets[i % 6][1]), args.steps, args.warmup)
@@ -511,6 +534,18 @@ def main():
             line["others"] = bench_others(ext, dev, args.steps, args.warmup, decode_calls=args.decode_calls)
         except Exception as e:                                      # keep the headline line intact
             line["others"] = {"error": repr(e)}
+        # The decode step's fractions beside the headline's: events over 400 warm launches, the same
+        # over 40 rotating buffer sets, and the device-side duration imported from the committed trace.
+        dec = {}
+        for key, name in (("update_linear_s3", "linear_s3"), ("update_circular_s8", "circular_s8")):
+            r = line["others"].get(key)
+            if isinstance(r, dict):
+                dec[name] = {"frac": r["frac_of_hbm_peak"], "frac_rotated": r.get("frac_of_hbm_peak_rotated"),
+                             "frac_device": round(gbs(r["algorithmic_bytes"], r["us_device_rocprof"]) / HBM_PEAK_GBS, 4)
+                                            if "us_device_rocprof" in r else None,
+                             "us": r["us"], "us_rotated": r.get("us_rotated")}
+        if dec:
+            line["roofline"]["decode"] = dec
     print(json.dumps(line), flush=True)
 
 

@@ -96,8 +96,15 @@ def run_under_rocprof(trace_dir, argv):
         elif not arg.startswith("--rocprof="):
             child_args.append(arg)
     os.makedirs(trace_dir, exist_ok=True)
+    # The program after `--` is this interpreter's own binary: a `python3` found on PATH may be a
+    # shim or a script that starts the real interpreter by exec, after rocprofv3's preloaded
+    # library has already initialised the GPU in it.
+    interpreter = os.path.realpath(sys.executable)
+    with open(interpreter, "rb") as f:
+        if f.read(4) != b"\x7fELF":
+            sys.exit("--rocprof: %s is not an ELF binary; rocprofv3 must start the interpreter itself" % interpreter)
     cmd = ["rocprofv3", "--kernel-trace", "--stats", "-d", trace_dir, "-o", "benchmark_ops", "--",
-           "python3", os.path.abspath(__file__)] + child_args
+           interpreter, os.path.abspath(__file__)] + child_args
     print("+ " + " ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0:

@@ -14,7 +14,6 @@
 #include <c10/hip/HIPStream.h>
 
 #include <cstdint>
-#include <cstdlib>
 #include <optional>
 
 #include "cc1d.h"
@@ -46,28 +45,18 @@ void check_status(int st, const char *op) {
 
 // The stream the launches go to: torch's current one.  A stream that is being captured into a
 // HIP graph is refused.  Nothing on the launch path allocates, clears memory or synchronises the
-// host, so capture ought to work, but it is not verified: the one capture run of these operators
+// host, so capture ought to work, but it is not verified: the two capture runs of these operators
 // (a decode loop, and a forward + backward, under torch.cuda.graph on a side stream) ended in a
 // segmentation fault on the host whose cause was never established, and an error that says so
-// is better than a crash in a serving process.  CC1D_ALLOW_GRAPH_CAPTURE=1 in the environment
-// lets the launches through for whoever wants to try.
-bool capture_allowed() {
-    static const bool allowed = [] {
-        const char *v = std::getenv("CC1D_ALLOW_GRAPH_CAPTURE");
-        return v != nullptr && v[0] != '\0' && v[0] != '0';
-    }();
-    return allowed;
-}
-
+// is better than a crash in a serving process.
 cc1d_stream_t current_stream() {
     hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
-    if (stream != nullptr && !capture_allowed()) {
+    if (stream != nullptr) {
         hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
         const hipError_t err = hipStreamIsCapturing(stream, &status);
         TORCH_CHECK(err == hipSuccess && status == hipStreamCaptureStatusNone,
                     "causal_conv1d: the current stream is being captured into a HIP graph; graph capture of "
-                    "these operators is not verified in this build (set CC1D_ALLOW_GRAPH_CAPTURE=1 to launch "
-                    "anyway)");
+                    "these operators is not verified in this build and is refused");
     }
     return static_cast<cc1d_stream_t>(stream);
 }

@@ -150,16 +150,33 @@ cc1d_update_params batch_slice(const cc1d_update_params &p, int b0, int n) {
     return q;
 }
 
-// launch(params) for the whole batch, or for halves of it (recursively) while it answers
-// CC1D_ERR_TOO_LARGE.  Slices run in batch order.
+// launch(params) for halves of the batch (recursively) while it answers CC1D_ERR_TOO_LARGE.
+// Slices run in batch order.
+template <typename P, typename F>
+int launch_halves(const P &p, F &&launch) {
+    const int st = launch(p);
+    if (st != CC1D_ERR_TOO_LARGE || p.batch < 2) return st;
+    const int head = p.batch / 2;
+    const int first = launch_halves(batch_slice(p, 0, head), launch);
+    if (first != CC1D_OK) return first;
+    return launch_halves(batch_slice(p, head, p.batch - head), launch);
+}
+
+// launch(params) for the whole batch or, when that answers CC1D_ERR_TOO_LARGE, in slices.  Whether
+// slicing can succeed is settled before the first slice runs: a launcher is asked, in probe mode,
+// about a single batch entry (the smallest slice the halving can end in; a problem whose launch
+// size does not shrink with the batch fails here), so an error leaves every output untouched
+// instead of partly written.
 template <typename P, typename F>
 int launch_in_batch_slices(const P &p, F &&launch) {
     const int st = launch(p);
     if (st != CC1D_ERR_TOO_LARGE || p.batch < 2) return st;
-    const int head = p.batch / 2;
-    const int first = launch_in_batch_slices(batch_slice(p, 0, head), launch);
-    if (first != CC1D_OK) return first;
-    return launch_in_batch_slices(batch_slice(p, head, p.batch - head), launch);
+    {
+        ProbeScope probe;
+        const int one = launch(batch_slice(p, 0, 1));
+        if (one != CC1D_OK) return one;
+    }
+    return launch_halves(p, launch);
 }
 
 size_t bwd_workspace_one_launch(const cc1d_bwd_params &p) {

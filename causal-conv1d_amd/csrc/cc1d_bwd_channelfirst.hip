@@ -932,40 +932,40 @@ int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStr
     const uint32_t blocks = (uint32_t)((waves + (kBlock / kWave) - 1) / (kBlock / kWave));
     if (g.streaming == 3) {                           // short rows, several batch entries to a wavefront
         switch (p.width) {
-            case 2: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 2, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            case 3: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 3, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            default: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 4, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 2: CC1D_LAUNCH((bwd_channelfirst_short_kernel<DT, 2, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: CC1D_LAUNCH((bwd_channelfirst_short_kernel<DT, 3, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: CC1D_LAUNCH((bwd_channelfirst_short_kernel<DT, 4, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         }
         return launch_status();
     }
     if (g.streaming == 4) {                           // the same, rows of any length anywhere in memory
         switch (p.width) {
-            case 2: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 2, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            case 3: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 3, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            default: hipLaunchKernelGGL((bwd_channelfirst_short_kernel<DT, 4, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 2: CC1D_LAUNCH((bwd_channelfirst_short_kernel<DT, 2, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: CC1D_LAUNCH((bwd_channelfirst_short_kernel<DT, 3, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: CC1D_LAUNCH((bwd_channelfirst_short_kernel<DT, 4, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         }
         return launch_status();
     }
     if (g.streaming == 1) {                           // rows on the grid, whole vectors
         switch (p.width) {
-            case 2: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 2, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            case 3: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 3, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            default: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 4, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 2: CC1D_LAUNCH((bwd_channelfirst_stream_kernel<DT, 2, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: CC1D_LAUNCH((bwd_channelfirst_stream_kernel<DT, 3, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: CC1D_LAUNCH((bwd_channelfirst_stream_kernel<DT, 4, false>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         }
         return launch_status();
     }
     if (g.streaming == 2) {                           // rows anywhere on the grid
         switch (p.width) {
-            case 2: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 2, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            case 3: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 3, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-            default: hipLaunchKernelGGL((bwd_channelfirst_stream_kernel<DT, 4, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 2: CC1D_LAUNCH((bwd_channelfirst_stream_kernel<DT, 2, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            case 3: CC1D_LAUNCH((bwd_channelfirst_stream_kernel<DT, 3, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+            default: CC1D_LAUNCH((bwd_channelfirst_stream_kernel<DT, 4, true>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
         }
         return launch_status();
     }
     switch (p.width) {
-        case 2: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-        case 3: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
-        default: hipLaunchKernelGGL((bwd_channelfirst_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        case 2: CC1D_LAUNCH((bwd_channelfirst_kernel<DT, 2>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        case 3: CC1D_LAUNCH((bwd_channelfirst_kernel<DT, 3>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
+        default: CC1D_LAUNCH((bwd_channelfirst_kernel<DT, 4>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws); break;
     }
     return launch_status();
 }

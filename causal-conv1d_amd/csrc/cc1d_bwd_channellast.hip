@@ -52,7 +52,7 @@ bwd_finalize_kernel(const float *__restrict__ ws, int n_parts, int dim, int widt
 int launch_bwd_finalize(const float *ws, int n_parts, const cc1d_bwd_params &p, hipStream_t stream) {
     const uint32_t planes = (uint32_t)p.width + (p.dbias != nullptr ? 1u : 0u);
     const uint32_t cblocks = ((uint32_t)p.dim + kFinChannels - 1) / kFinChannels;
-    hipLaunchKernelGGL(bwd_finalize_kernel, dim3(planes * cblocks), dim3(kFinSlices * kFinChannels), 0, stream,
+    CC1D_LAUNCH(bwd_finalize_kernel, dim3(planes * cblocks), dim3(kFinSlices * kFinChannels), 0, stream,
                        ws, n_parts, p.dim, p.width, p.dweight, p.dw_stride_c, p.dw_stride_w, p.dbias,
                        p.overwrite_dweight);
     return launch_status();

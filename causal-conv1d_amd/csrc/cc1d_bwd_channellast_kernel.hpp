@@ -476,9 +476,9 @@ int launch_instance(const cc1d_bwd_params &p, const BwdClGeom &g, float *ws, hip
     constexpr int U = CC1D_BWD_CL_UNROLL;
     const uint32_t blocks = g.blocks_per_xcd * kXcds;
     if (p.silu)
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
+        CC1D_LAUNCH((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
     else
-        hipLaunchKernelGGL((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
+        CC1D_LAUNCH((bwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>), dim3(blocks), dim3(kBlock), 0, stream, p, g, ws, p.seq_idx);
     return launch_status();
 }
 

@@ -567,9 +567,9 @@ int launch_short(const cc1d_fwd_params &p, int n_vecs, bool aligned, hipStream_t
     const uint32_t n_rows = (uint32_t)rows;
     const bool batch_inner = batch_entries_are_neighbours(p);
 #define CC1D_SHORT3(WIDTH, SILU_ON, BI_ON)                                                                           \
-    if (aligned) hipLaunchKernelGGL((fwd_channelfirst_short_kernel<DT, WIDTH, SILU_ON, true, BI_ON>), grid, block, 0, \
+    if (aligned) CC1D_LAUNCH((fwd_channelfirst_short_kernel<DT, WIDTH, SILU_ON, true, BI_ON>), grid, block, 0, \
                                     stream, p, n_vecs, lanes_log2, n_rows);                                           \
-    else hipLaunchKernelGGL((fwd_channelfirst_short_kernel<DT, WIDTH, SILU_ON, false, BI_ON>), grid, block, 0,       \
+    else CC1D_LAUNCH((fwd_channelfirst_short_kernel<DT, WIDTH, SILU_ON, false, BI_ON>), grid, block, 0,       \
                             stream, p, n_vecs, lanes_log2, n_rows)
 #define CC1D_SHORT2(WIDTH, SILU_ON)                                                                                  \
     if (batch_inner) { CC1D_SHORT3(WIDTH, SILU_ON, true); } else { CC1D_SHORT3(WIDTH, SILU_ON, false); }
@@ -728,9 +728,9 @@ int launch_flat(const cc1d_fwd_params &p, hipStream_t stream) {
     const dim3 grid((n_vecs + kBlock - 1) / kBlock), block(kBlock);
     const bool packed = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
 #define CC1D_FLAT2(WIDTH, SILU_ON)                                                                                    \
-    if (packed) hipLaunchKernelGGL((fwd_channelfirst_flat_kernel<DT, WIDTH, SILU_ON, true>), grid, block, 0, stream,  \
+    if (packed) CC1D_LAUNCH((fwd_channelfirst_flat_kernel<DT, WIDTH, SILU_ON, true>), grid, block, 0, stream,  \
                                    p, n_elems);                                                                       \
-    else hipLaunchKernelGGL((fwd_channelfirst_flat_kernel<DT, WIDTH, SILU_ON, false>), grid, block, 0, stream, p,     \
+    else CC1D_LAUNCH((fwd_channelfirst_flat_kernel<DT, WIDTH, SILU_ON, false>), grid, block, 0, stream, p,     \
                             n_elems)
 #define CC1D_FLAT(WIDTH)                                                                                              \
     if (p.silu) { CC1D_FLAT2(WIDTH, true); } else { CC1D_FLAT2(WIDTH, false); }
@@ -748,9 +748,9 @@ template <int DT, bool SILU, int U, bool BI>
 int launch_stream(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t stream) {
     const uint32_t blocks = (g.total_waves + (kBlock / kWave) - 1) / (kBlock / kWave);
     switch (p.width) {
-        case 2: hipLaunchKernelGGL((fwd_channelfirst_stream_kernel<DT, 2, SILU, U, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
-        case 3: hipLaunchKernelGGL((fwd_channelfirst_stream_kernel<DT, 3, SILU, U, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
-        default: hipLaunchKernelGGL((fwd_channelfirst_stream_kernel<DT, 4, SILU, U, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        case 2: CC1D_LAUNCH((fwd_channelfirst_stream_kernel<DT, 2, SILU, U, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        case 3: CC1D_LAUNCH((fwd_channelfirst_stream_kernel<DT, 3, SILU, U, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        default: CC1D_LAUNCH((fwd_channelfirst_stream_kernel<DT, 4, SILU, U, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
     }
     return launch_status();
 }
@@ -761,9 +761,9 @@ int launch_order(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t strea
     if (g.streaming == 1) return p.silu ? launch_stream<DT, true, 1, BI>(p, g, stream) : launch_stream<DT, false, 1, BI>(p, g, stream);
     const uint32_t blocks = (g.total_waves + (kBlock / kWave) - 1) / (kBlock / kWave);
     switch (p.width) {
-        case 2: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 2, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
-        case 3: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 3, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
-        default: hipLaunchKernelGGL((fwd_channelfirst_kernel<DT, 4, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        case 2: CC1D_LAUNCH((fwd_channelfirst_kernel<DT, 2, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        case 3: CC1D_LAUNCH((fwd_channelfirst_kernel<DT, 3, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
+        default: CC1D_LAUNCH((fwd_channelfirst_kernel<DT, 4, BI>), dim3(blocks), dim3(kBlock), 0, stream, p, g); break;
     }
     return launch_status();
 }
@@ -810,7 +810,7 @@ int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
         // lane that reads a row's initial_states and the lane that writes its final_states can sit in
         // different wavefronts.)
         const bool states_in_and_out = p.initial_states != nullptr && p.final_states != nullptr;
-        const bool flat = !aligned && !states_in_and_out && p.seqlen >= vec && n_elems < ((int64_t)1 << 31) &&
+        const bool flat = !aligned && !states_in_and_out && p.seqlen >= vec && n_elems < thread_limit() &&
                           aligned16(p.x) && aligned16(p.out) &&
                           (p.dim == 1 || (p.x_stride_c == p.seqlen && p.out_stride_c == p.seqlen)) &&
                           (p.batch == 1 || (p.x_stride_b == (int64_t)p.dim * p.seqlen &&

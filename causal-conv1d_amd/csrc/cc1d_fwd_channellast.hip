@@ -441,10 +441,10 @@ int launch_instance(const cc1d_fwd_params &p, const FwdClGeom &g, const VarlenTa
     constexpr int U = CC1D_FWD_CL_UNROLL;
     const uint32_t blocks = tail.first_block + (tail.total + kBlock - 1) / kBlock;
     if (p.silu)
-        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>),
+        CC1D_LAUNCH((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, true, U, WM>),
                            dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx, tail);
     else
-        hipLaunchKernelGGL((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>),
+        CC1D_LAUNCH((fwd_channellast_kernel<DT, CH, W, HAS_SEQ, false, U, WM>),
                            dim3(blocks), dim3(kBlock), 0, stream, p, g, p.seq_idx, tail);
     return launch_status();
 }

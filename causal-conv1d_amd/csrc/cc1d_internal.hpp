@@ -79,7 +79,23 @@ inline int64_t thread_limit() {
 }
 inline int64_t wave_limit() { return thread_limit() / 64; }
 
+// Probe mode, per host thread: a launcher called in it does everything it does before a launch
+// (layout choice, geometry, the checks that answer CC1D_ERR_TOO_LARGE) and launches nothing.  The
+// C-ABI front uses it to learn whether the smallest batch slice of a problem fits one grid before
+// the first slice is launched.
+inline thread_local bool g_probe_only = false;
+inline bool probe_only() { return g_probe_only; }
+struct ProbeScope {
+    ProbeScope() { g_probe_only = true; }
+    ~ProbeScope() { g_probe_only = false; }
+};
+#define CC1D_LAUNCH(...)                                            \
+    do {                                                            \
+        if (!::cc1d::probe_only()) hipLaunchKernelGGL(__VA_ARGS__); \
+    } while (0)
+
 inline int launch_status() {
+    if (probe_only()) return CC1D_OK;
     return hipGetLastError() == hipSuccess ? CC1D_OK : CC1D_ERR_LAUNCH;
 }
 

@@ -727,14 +727,15 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         a.n_colgroups = (uint32_t)(p.dim / CH);
         const dim3 grid((a.n_colgroups + kWave - 1) / kWave,
                         (uint32_t)((p.batch + kStepWaves * kStepRows - 1) / (kStepWaves * kStepRows)));
+        if ((int64_t)grid.x * grid.y * kBlock >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         auto launch = [&](auto wm) {
             constexpr int WM = decltype(wm)::value;
             if (circ) {
-                if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, true, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
-                else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, true, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+                if (p.silu) CC1D_LAUNCH((update_step_kernel<DT, CH, W, true, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+                else CC1D_LAUNCH((update_step_kernel<DT, CH, W, true, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
             } else {
-                if (p.silu) hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
-                else hipLaunchKernelGGL((update_step_kernel<DT, CH, W, false, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+                if (p.silu) CC1D_LAUNCH((update_step_kernel<DT, CH, W, false, true, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
+                else CC1D_LAUNCH((update_step_kernel<DT, CH, W, false, false, kStepRows, WM>), grid, dim3(kBlock), 0, stream, a);
             }
         };
         if (mode == 1) launch(std::integral_constant<int, 1>{});
@@ -758,14 +759,15 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         a.n_colgroups = (uint32_t)(p.dim / CH);
         ta.x_stride_l = p.x_stride_l; ta.out_stride_l = p.out_stride_l; ta.seqlen = p.seqlen;
         const dim3 grid((a.n_colgroups + kWave - 1) / kWave, (uint32_t)((p.batch + kStepWaves - 1) / kStepWaves));
+        if ((int64_t)grid.x * grid.y * kBlock >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         auto launch = [&](auto wm) {
             constexpr int WM = decltype(wm)::value;
             if (circ) {
-                if (p.silu) hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, true, true, WM>), grid, dim3(kBlock), 0, stream, ta);
-                else hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, true, false, WM>), grid, dim3(kBlock), 0, stream, ta);
+                if (p.silu) CC1D_LAUNCH((update_tokens_kernel<DT, CH, W, true, true, WM>), grid, dim3(kBlock), 0, stream, ta);
+                else CC1D_LAUNCH((update_tokens_kernel<DT, CH, W, true, false, WM>), grid, dim3(kBlock), 0, stream, ta);
             } else {
-                if (p.silu) hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, false, true, WM>), grid, dim3(kBlock), 0, stream, ta);
-                else hipLaunchKernelGGL((update_tokens_kernel<DT, CH, W, false, false, WM>), grid, dim3(kBlock), 0, stream, ta);
+                if (p.silu) CC1D_LAUNCH((update_tokens_kernel<DT, CH, W, false, true, WM>), grid, dim3(kBlock), 0, stream, ta);
+                else CC1D_LAUNCH((update_tokens_kernel<DT, CH, W, false, false, WM>), grid, dim3(kBlock), 0, stream, ta);
             }
         };
         if (mode == 1) launch(std::integral_constant<int, 1>{});
@@ -777,7 +779,7 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
     // lane's accesses to the state, x and out are aligned.
     if (p.seqlen == 1 && !circ && p.state_stride_l == 1 && p.state_stride_c == p.state_len && p.x_stride_c == 1 &&
         p.out_stride_c == 1 && p.state_len >= W - 1 && p.batch <= 65535 * kStepWaves) {
-        bool launched = false;
+        bool launched = false, too_large = false;
         auto run = [&](auto sc) {
             constexpr int SC = decltype(sc)::value;
             if constexpr (SC >= W - 1) {
@@ -795,21 +797,22 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
                      !rows_lane_ok(p.out, DT, kLaneBytes, p.out_stride_b, 1, 0, 1))) return;
                 const uint32_t n_groups = (uint32_t)(p.dim / CHC);
                 const dim3 grid((n_groups + kWave - 1) / kWave, (uint32_t)((p.batch + kStepWaves - 1) / kStepWaves));
+                if ((int64_t)grid.x * grid.y * kBlock >= thread_limit()) { too_large = true; return; }
                 const int w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
                 constexpr bool kStage32 = CHC % 2 == 0;
                 constexpr bool kStage16 = DT != CC1D_F32 && CHC % 4 == 0;
                 constexpr bool kLane16 = DT != CC1D_F32 && CHC % 2 == 0 && !kStage16;
                 if (mode == 1 && kStage32) {
                     if constexpr (kStage32)
-                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 1>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                        CC1D_LAUNCH((update_rowstate_kernel<DT, W, SC, CHC, VB, 1>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
                 } else if (mode == 2 && kStage16) {
                     if constexpr (kStage16)
-                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 2>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                        CC1D_LAUNCH((update_rowstate_kernel<DT, W, SC, CHC, VB, 2>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
                 } else if (mode == 2 && kLane16) {
                     if constexpr (kLane16)
-                        hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 3>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                        CC1D_LAUNCH((update_rowstate_kernel<DT, W, SC, CHC, VB, 3>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
                 } else {
-                    hipLaunchKernelGGL((update_rowstate_kernel<DT, W, SC, CHC, VB, 0>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
+                    CC1D_LAUNCH((update_rowstate_kernel<DT, W, SC, CHC, VB, 0>), grid, dim3(kBlock), 0, stream, p, n_groups, w_fast);
                 }
                 launched = true;
             }
@@ -821,6 +824,7 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
             case 8: run(std::integral_constant<int, 8>{}); break;
             default: break;
         }
+        if (too_large) return CC1D_ERR_TOO_LARGE;
         if (launched) return launch_status();
     }
     if (vec) {
@@ -829,14 +833,14 @@ int launch_w(const cc1d_update_params &p, bool vec, hipStream_t stream) {
         if (total >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
         const int w_fast = weights_contiguous_f32(p.weight, p.w_dtype, p.w_stride_c, p.w_stride_w, p.width);
-        if (circ) hipLaunchKernelGGL((update_vec_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, p, ncg, (uint32_t)total, w_fast);
-        else hipLaunchKernelGGL((update_vec_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, p, ncg, (uint32_t)total, w_fast);
+        if (circ) CC1D_LAUNCH((update_vec_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, p, ncg, (uint32_t)total, w_fast);
+        else CC1D_LAUNCH((update_vec_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, p, ncg, (uint32_t)total, w_fast);
     } else {
         const int64_t total = (int64_t)p.batch * p.dim;
         if (total >= thread_limit()) return CC1D_ERR_TOO_LARGE;
         const uint32_t blocks = (uint32_t)((total + kBlock - 1) / kBlock);
-        if (circ) hipLaunchKernelGGL((update_generic_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, p, (uint32_t)total);
-        else hipLaunchKernelGGL((update_generic_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, p, (uint32_t)total);
+        if (circ) CC1D_LAUNCH((update_generic_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, p, (uint32_t)total);
+        else CC1D_LAUNCH((update_generic_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, p, (uint32_t)total);
     }
     return launch_status();
 }

@@ -44,12 +44,12 @@ int launch_dtype(const cc1d_varlen_params &p, bool vec, hipStream_t stream) {
         const uint32_t ncg = (uint32_t)(p.dim / Elem<DT>::kVec);
         const int64_t total = (int64_t)p.batch * p.state_len * ncg;
         if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
-        hipLaunchKernelGGL((varlen_states_vec_kernel<DT>), dim3((uint32_t)((total + kBlock - 1) / kBlock)),
+        CC1D_LAUNCH((varlen_states_vec_kernel<DT>), dim3((uint32_t)((total + kBlock - 1) / kBlock)),
                            dim3(kBlock), 0, stream, p, ncg, (uint32_t)total);
     } else {
         const int64_t total = (int64_t)p.batch * p.state_len * p.dim;
         if (total >= ((int64_t)1 << 31)) return CC1D_ERR_TOO_LARGE;
-        hipLaunchKernelGGL((varlen_states_elem_kernel<DT>), dim3((uint32_t)((total + kBlock - 1) / kBlock)),
+        CC1D_LAUNCH((varlen_states_elem_kernel<DT>), dim3((uint32_t)((total + kBlock - 1) / kBlock)),
                            dim3(kBlock), 0, stream, p, (uint32_t)total);
     }
     return launch_status();

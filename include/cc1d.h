@@ -154,8 +154,9 @@ int cc1d_bwd_workspace_bytes(const cc1d_bwd_params *p, size_t *bytes);
 int cc1d_bwd(const cc1d_bwd_params *p, void *workspace, size_t workspace_bytes,
              cc1d_stream_t stream);
 
-/* The backward for callers that cannot allocate device memory: code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference, whose
+/* The backward for callers that cannot allocate device memory: tight serving loops, harnesses
+ * that forbid hipMalloc, code that is to be captured into a HIP graph (capture itself has not been
+ * verified with this library; what this entry point guarantees is that it allocates nothing).  No counterpart in the reference, whose
  * backward allocates its workspaces itself with at::zeros (csrc/causal_conv1d.cpp:396-429).
  * Same kernels, same order of additions and same results as cc1d_bwd; the partial-sum workspace
  * is a fixed array of CC1D_BWD_NOALLOC_MAX_WORKSPACE_BYTES inside this library's device image
@@ -168,7 +169,7 @@ int cc1d_bwd(const cc1d_bwd_params *p, void *workspace, size_t workspace_bytes,
  * overlap in time on one GPU (different streams, no ordering between them) race; calls on one
  * stream never do.  The array needs no clearing between calls (every plane that is read was
  * written by the same call).  The first call on a device looks the array's address up
- * (hipGetSymbolAddress), so make it outside graph capture. */
+ * (hipGetSymbolAddress): make that call before any stream of the device is being captured. */
 #define CC1D_BWD_NOALLOC_MAX_WORKSPACE_BYTES (16u * 1024u * 1024u)
 int cc1d_bwd_noalloc(const cc1d_bwd_params *p, cc1d_stream_t stream);
 
