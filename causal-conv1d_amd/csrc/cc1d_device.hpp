@@ -295,7 +295,7 @@ struct PackedTaps {
     static constexpr int kBiasWords = k32 ? NCH : NCH / 2;
     uint32_t wraw[kWords];
     uint32_t braw[kBiasWords];
-    static_assert(NCH % 2 == 0, "two 16-bit taps per word");
+    static_assert(k32 || NCH % 2 == 0, "two 16-bit taps per word");
 
     static constexpr int pow2_align(int bytes) { return bytes % 16 == 0 ? 16 : bytes % 8 == 0 ? 8 : 4; }
 
