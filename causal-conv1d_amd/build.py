@@ -71,6 +71,20 @@ def _newer(target, deps):
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
+def compile_command(src, obj, extra_flags=()):
+    """The hipcc command line that turns one source of csrc/ into an object with gfx950 device code."""
+    s = os.path.join(CSRC, src)
+    lang = ["-x", "hip"] if src.endswith(".cpp") else []
+    return [HIPCC] + HIP_FLAGS + list(extra_flags) + lang + ["-c", s, "-o", obj]
+
+
+def compile_source(src, obj, extra_flags=()):
+    """Compile one source of csrc/ (always: no up-to-date check)."""
+    os.makedirs(os.path.dirname(obj), exist_ok=True)
+    _run(compile_command(src, obj, extra_flags))
+    return obj
+
+
 def build_kernels(force=False, extra_flags=(), lib_path=None):
     """Compile every HIP source for gfx950 and link libcc1d.so."""
     os.makedirs(OBJDIR, exist_ok=True)
@@ -83,8 +97,7 @@ def build_kernels(force=False, extra_flags=(), lib_path=None):
         o = os.path.join(OBJDIR, os.path.splitext(src)[0] + tag + ".o")
         objs.append(o)
         if force or not _newer(o, [s] + headers):
-            lang = ["-x", "hip"] if src.endswith(".cpp") else []
-            jobs.append([HIPCC] + HIP_FLAGS + list(extra_flags) + lang + ["-c", s, "-o", o])
+            jobs.append(compile_command(src, o, extra_flags))
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         list(ex.map(_run, jobs))
     if force or jobs or not _newer(lib_path, objs):
@@ -98,13 +111,15 @@ def build_kernels(force=False, extra_flags=(), lib_path=None):
     return lib_path
 
 
-def build_binding(force=False):
-    """Compile the host-only torch binding with g++ and link it against libcc1d.so."""
+def build_binding(force=False, out_dir=None):
+    """Compile the host-only torch binding with g++ and link it against libcc1d.so.  `out_dir`:
+    where the extension module goes (default: next to this file, beside libcc1d.so, which the
+    module looks for in its own directory)."""
     from torch.utils import cpp_extension as ce
     import torch
 
     src = os.path.join(CSRC, "causal_conv1d.cpp")
-    out = os.path.join(HERE, EXT_NAME)
+    out = os.path.join(out_dir or HERE, EXT_NAME)
     if not force and _newer(out, [src, os.path.join(INCLUDE, "cc1d.h")]):
         return out
     cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",

@@ -30,6 +30,30 @@ print("installed copy ok")
 """
 
 
+def test_build_step_compiles_device_code_and_binding(cc1d_lib, tmp_path):
+    """The two tests below install what build.py has already built in the tree (up-to-date objects
+    are not recompiled).  This one makes the build step compile: one kernel source into a fresh
+    object, which must hold a gfx950 code object, and the torch binding into a fresh directory,
+    which must import from there beside a copy of the kernel library."""
+    import shutil
+    import time
+    sys.path.insert(0, PKG_DIR)
+    import build as cc1d_build
+    started = time.time()
+    obj = cc1d_build.compile_source("cc1d_varlen_states.hip", str(tmp_path / "obj" / "cc1d_varlen_states.o"))
+    assert os.path.getmtime(obj) >= started - 1.0
+    blob = open(obj, "rb").read()
+    assert blob[:4] == b"\x7fELF" and b"gfx950" in blob and b"varlen_states" in blob
+    site = str(tmp_path / "site")
+    os.makedirs(site)
+    ext = cc1d_build.build_binding(force=True, out_dir=site)
+    assert os.path.dirname(ext) == site and os.path.getmtime(ext) >= started - 1.0
+    shutil.copy2(os.path.join(PKG_DIR, cc1d_build.LIB_NAME), site)
+    shutil.copytree(os.path.join(PKG_DIR, "causal_conv1d"), os.path.join(site, "causal_conv1d"),
+                    ignore=shutil.ignore_patterns("__pycache__"))
+    _check_installed(site)
+
+
 def _check_installed(site):
     env = {k: v for k, v in os.environ.items() if k != "PYTHONPATH"}
     env["PYTHONPATH"] = site
