@@ -27,10 +27,12 @@ KERNEL_SOURCES = [
     "cc1d_api.cpp",
     "cc1d_fwd_channellast.hip",
     "cc1d_fwd_channelfirst.hip",
+    "cc1d_fwd_channelfirst_tile.hip",
     "cc1d_bwd_channellast.hip",
     "cc1d_bwd_channellast_lanes4.hip",
     "cc1d_bwd_channellast_lanes8.hip",
     "cc1d_bwd_channelfirst.hip",
+    "cc1d_bwd_channelfirst_tile.hip",
     "cc1d_bwd_noalloc.hip",
     "cc1d_update.hip",
     "cc1d_varlen_states.hip",

@@ -972,19 +972,32 @@ int launch_dtype(const cc1d_bwd_params &p, const BwdCfGeom &g, float *ws, hipStr
 
 }  // namespace
 
+// Rows of more than 64 vectors take the tile kernel (a forced number of parts keeps them on the
+// walking kernels above).
+static bool takes_tiles(const cc1d_bwd_params &p) {
+    return tunables().bwd_cf_parts == 0 && bwd_channelfirst_tile_applies(p);
+}
+
 size_t bwd_channelfirst_workspace_bytes(const cc1d_bwd_params &p) {
+    if (takes_tiles(p)) return (size_t)bwd_channelfirst_tile_parts(p) * (p.width + 1) * (size_t)p.dim * sizeof(float);
     const BwdCfGeom g = make_geom(p);
     if (g.n_parts == 1) return 0;
     return (size_t)g.n_parts * (p.width + 1) * (size_t)p.dim * sizeof(float);
 }
 
 bool bwd_channelfirst_fits(const cc1d_bwd_params &p) {
+    if (takes_tiles(p)) return bwd_channelfirst_tile_fits(p);
     return (int64_t)p.dim * make_geom(p).n_parts < wave_limit();
 }
 
 int launch_bwd_channelfirst(const cc1d_bwd_params &p, void *workspace, hipStream_t stream) {
-    const BwdCfGeom g = make_geom(p);
     float *ws = static_cast<float *>(workspace);
+    if (takes_tiles(p)) {
+        const int st = launch_bwd_channelfirst_tile(p, ws, stream);
+        if (st != CC1D_OK) return st;
+        return launch_bwd_finalize(ws, bwd_channelfirst_tile_parts(p), p, stream);
+    }
+    const BwdCfGeom g = make_geom(p);
     int st;
     switch (p.x_dtype) {
         case CC1D_F32: st = launch_dtype<CC1D_F32>(p, g, ws, stream); break;

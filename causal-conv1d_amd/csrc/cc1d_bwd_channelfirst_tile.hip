@@ -1,0 +1,346 @@
+// Channel-first backward for gfx950, rows longer than 64 vectors: short-lived tile wavefronts.
+// Takes over causal_conv1d_bwd_kernel (csrc/causal_conv1d_bwd.cu:53-259 of the reference) for
+// these rows; formulas as in cc1d_bwd_channelfirst.hip, whose kernels keep the short rows.
+//
+//   z[t]  = bias + sum_w weight[w] * xpad[t-(W-1-w)]
+//   g[t]  = dout[t] * act'(z[t])
+//   dx[p] = sum_k weight[W-1-k] * g[p+k]   (+ dfinal_states[p-(L-(W-1))] for p >= L-(W-1))
+//   dinitial_states[i] = the same expression at p = i-(W-1) < 0
+//   dweight[w] += sum_{b,t} g[t] * xpad[t-(W-1-w)],   dbias += sum_{b,t} g[t]
+//
+// Design.  A wavefront takes a tile of up to four 64-vector steps of one (batch, channel) row
+// and asks for all of its x and dout at once; the data goes from memory straight into LDS
+// (buffer_load_dwordx4 ... lds) together with the vector in front of the tile (the x halo) and
+// the vectors behind it (x and dout of the W-1 positions whose g the tile's last lane needs).
+// No registers are held while the tile is in flight, so the launch is thousands of wavefronts
+// that live for one memory round trip and a few hundred instructions each and sweep through
+// memory as one compact front in the order of the rows -- where one long-lived wavefront per
+// channel walks 4096 far-apart streams at once, which is what bounds that design at the
+// backward's benchmark shape (fp16 (4, 4096, 8192): 141 us for its memory pattern alone,
+// 122 us for this one).  Each of the three tensors is a buffer resource per row, based at the
+// row's first element wherever that lies (the vector accesses need no alignment, so rows of any
+// length anywhere in memory take the same path: (16, 4096, 1001) bf16 costs 4 % more than 1000
+// where the walking kernel took 2.2 times as long), and what lies outside a row needs no test:
+// the vector in front of the first tile and everything behind the row's end is out of range,
+// reads as zero and is not stored.  A 16-bit row of odd length ends in half a dword, which the
+// range check would drop: that one element is fetched and stored on its own.
+// The steps of a tile are computed top down.  A lane's x halo is the upper half of the previous
+// vector in LDS; the g values to the right of its vector come from the next lane (DPP shift),
+// for the last lane from the step above (carried), for the top step from the vectors behind the
+// tile.  The lane's dweight / dbias terms stay in registers across the tile, are reduced over
+// the 64 lanes in a fixed order (DPP) and stored as one workspace plane per (batch entry, tile);
+// the second-stage kernel shared with the other backward kernels adds the planes in a fixed
+// order: no atomics, bit-reproducible.
+#include <type_traits>
+
+#include "cc1d_device.hpp"
+#include "cc1d_internal.hpp"
+
+namespace cc1d {
+namespace {
+
+constexpr int kTileSteps = 4;                     // 64-vector steps per tile
+constexpr int kTileVecs = kTileSteps * kWave;     // 256 vectors, 4 KiB per tensor
+constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
+
+typedef void __attribute__((address_space(3))) *lds_ptr_t;
+
+struct BwdCfTileArgs {
+    uint32_t total;               // rows * tiles_per_row wavefronts
+    uint32_t tiles_per_row;
+    int32_t seqlen;
+    int32_t batch, dim;
+    int32_t batch_inner;          // rows numbered with the batch entry fastest
+    int32_t w_dtype;
+    const void *x;
+    const void *dout;
+    void *dx;
+    const void *weight;
+    const void *bias;
+    float *ws;                    // [batch * tiles_per_row][W + 1][dim]
+    int64_t x_stride_b, x_stride_c, dout_stride_b, dout_stride_c, dx_stride_b, dx_stride_c;   // elements
+    int64_t w_stride_c, w_stride_w;
+    const void *initial_states;
+    const void *dfinal_states;
+    void *dinitial_states;
+    int64_t init_stride_b, init_stride_c, init_stride_l;
+    int64_t dfinal_stride_b, dfinal_stride_c, dfinal_stride_l;
+    int64_t dinit_stride_b, dinit_stride_c, dinit_stride_l;
+};
+
+// Sum over the 64 lanes in a fixed order, result in lane 63: prefix sums inside each row of 16
+// lanes (row_shr 1, 2, 4, 8), then the rows' totals across (row_bcast 15, 31).
+__device__ __forceinline__ float wave_total_in_lane63(float v) {
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x111, 0xf, 0xf, true));
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x112, 0xf, 0xf, true));
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x114, 0xf, 0xf, true));
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x118, 0xf, 0xf, true));
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x142, 0xa, 0xf, true));   // row_bcast:15 into rows 1, 3
+    v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x143, 0xc, 0xf, true));   // row_bcast:31 into rows 2, 3
+    return v;
+}
+
+template <int DT, int W, bool SILU>
+__global__ void __launch_bounds__(kBlock, 4)
+bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    constexpr int VEC = E::kVec;
+    constexpr int EB = E::kBytes;
+    constexpr bool PRECISE = E::kPreciseAct;
+    constexpr int XV = kTileVecs + 2, DV = kTileVecs + 1;     // vectors of x and of dout a tile holds
+    __shared__ u32x4 lds[kBlock / kWave][XV + DV];
+
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const int lane = (int)(threadIdx.x & (kWave - 1));
+    const uint32_t wid = blockIdx.x * (uint32_t)(kBlock / kWave) + (uint32_t)wv;
+    if (wid >= a.total) return;
+    const int tile = (int)(wid % a.tiles_per_row);
+    const uint32_t row = wid / a.tiles_per_row;
+    int b, c;
+    if (a.batch_inner) { b = (int)(row % (uint32_t)a.batch); c = (int)(row / (uint32_t)a.batch); }
+    else { c = (int)(row % (uint32_t)a.dim); b = (int)(row / (uint32_t)a.dim); }
+    const int L = a.seqlen;
+
+    const T *xrow = reinterpret_cast<const T *>(a.x) + (int64_t)b * a.x_stride_b + (int64_t)c * a.x_stride_c;
+    const T *drow = reinterpret_cast<const T *>(a.dout) + (int64_t)b * a.dout_stride_b + (int64_t)c * a.dout_stride_c;
+    T *dxrow = reinterpret_cast<T *>(a.dx) + (int64_t)b * a.dx_stride_b + (int64_t)c * a.dx_stride_c;
+    // The range check works on whole dwords: a 16-bit row of odd length ends in half a dword,
+    // which stays outside the resources; its element is moved separately below.
+    const int row_bytes = (L * EB) & ~3;
+    const bool odd_tail = ((L * EB) & 2) != 0;
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xrow), 0, row_bytes, kRsrcRaw);
+    const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(drow), 0, row_bytes, kRsrcRaw);
+    const __amdgpu_buffer_rsrc_t rdx = __builtin_amdgcn_make_buffer_rsrc(dxrow, 0, row_bytes, kRsrcRaw);
+    const int n_vecs = (L + VEC - 1) / VEC;
+    const int v0 = tile * kTileVecs;                  // the tile's first vector
+    int steps = (n_vecs - v0 + kWave - 1) / kWave;    // steps of the tile that reach into the row
+    steps = steps > kTileSteps ? kTileSteps : steps;
+    // x vector i of the wavefront's LDS holds row vector v0 - 1 + i, dout vector i holds v0 + i.
+    // For the row's first tile the x offset below wraps around: out of range, zeros.
+    u32x4 *xl = &lds[wv][0], *dl = &lds[wv][XV];
+    const int vx = (lane + v0 - 1) * 16, vd = (lane + v0) * 16;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 0, 2);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 0, 2);
+    if (steps > 1) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 1024, 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 1024, 2);
+    }
+    if (steps > 2) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 2048, 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 2048, 2);
+    }
+    if (steps > 3) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 3072, 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 3072, 2);
+    }
+    // behind the tile: two more vectors of x, one of dout (what the top step's last lane needs)
+    if (lane < 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(xl + steps * kWave), 16, vx + steps * 1024, 0, 0, 0);
+    if (lane < 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)(dl + steps * kWave), 16, vd + steps * 1024, 0, 0, 0);
+
+    // Taps and bias of the channel (wave-uniform); with the fast activation also times -log2(e),
+    // so that the sum over the window is the exponent the derivative needs.
+    float wv_[W], wvs[W], bias_v, bias_s;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+        wv_[w] = ld_weight(a.weight, a.w_dtype, (int64_t)c * a.w_stride_c + w * a.w_stride_w);
+    bias_v = a.bias == nullptr ? 0.f : ld_weight(a.bias, a.w_dtype, c);
+#pragma unroll
+    for (int w = 0; w < W; ++w) wvs[w] = wv_[w] * kSiluPrescale;
+    bias_s = bias_v * kSiluPrescale;
+
+    // What the resources leave out, fetched by single lanes: the odd last element of a 16-bit row
+    // (by the tile that holds it) and initial_states in front of the row (by its first tile).
+    const int tile_first = v0 * VEC, tile_end = (v0 + steps * kWave) * VEC;     // positions [tile_first, tile_end)
+    const bool holds_last = odd_tail && L - 1 >= tile_first - VEC && L - 1 < tile_end + VEC;
+    T last_x = T(0.f), last_d = T(0.f);
+    if (holds_last && lane == 0) {
+        last_x = ld_raw<DT>(xrow, L - 1);
+        last_d = ld_raw<DT>(drow, L - 1);
+    }
+    T init_raw[W - 1];
+    const bool has_init = a.initial_states != nullptr && tile == 0;
+    if (has_init && lane == 0) {
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i)
+            init_raw[i] = ld_raw<DT>(a.initial_states, (int64_t)b * a.init_stride_b + (int64_t)c * a.init_stride_c +
+                                                           (int64_t)i * a.init_stride_l);
+    }
+    // dfinal_states is added to the row's last W-1 positions: the tile that holds any of them
+    // fetches the values (wave-uniform), and only the steps that hold them look.
+    const bool has_dfinal = a.dfinal_states != nullptr && L - 1 >= tile_first && L - (W - 1) < tile_end;
+    float dfin[W - 1];
+#pragma unroll
+    for (int i = 0; i < W - 1; ++i) dfin[i] = 0.f;
+    if (has_dfinal) {
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i)
+            dfin[i] = ld_elem<DT>(a.dfinal_states, (int64_t)b * a.dfinal_stride_b + (int64_t)c * a.dfinal_stride_c +
+                                                       (int64_t)i * a.dfinal_stride_l);
+    }
+    // Every vector of the tile is in LDS behind this wait (a vector fetched into LDS counts as a
+    // load until it has been written there).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (holds_last && lane == 0) {
+        // LDS element index of row position p: x region (p + VEC - tile_first), dout region (p - tile_first)
+        const int ix = L - 1 + VEC - tile_first, id = L - 1 - tile_first;
+        if (ix >= 0 && ix < XV * VEC) reinterpret_cast<T *>(xl)[ix] = last_x;
+        if (id >= 0 && id < DV * VEC) reinterpret_cast<T *>(dl)[id] = last_d;
+    }
+    if (has_init && lane == 0) {
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i) reinterpret_cast<T *>(xl)[VEC - (W - 1) + i] = init_raw[i];
+    }
+
+    auto act_grad = [&](const float *xwin) { return silu_grad_of_window<W, PRECISE>(wv_, bias_v, wvs, bias_s, xwin); };
+    // g at the W-1 positions behind the tile, by every lane (the values are wave-uniform)
+    float carry[W - 1];
+    {
+        float xa[VEC], xb[VEC], dv[VEC];
+        E::unpack(xl[steps * kWave], xa);
+        E::unpack(xl[steps * kWave + 1], xb);
+        E::unpack(dl[steps * kWave], dv);
+        float xwin[2 * (W - 1)];
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i) { xwin[i] = xa[VEC - (W - 1) + i]; xwin[W - 1 + i] = xb[i]; }
+#pragma unroll
+        for (int e = 0; e < W - 1; ++e) carry[e] = SILU ? __builtin_fmaf(dv[e], act_grad(&xwin[e]), 0.f) : dv[e];
+    }
+    float dW[W], dB = 0.f;
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = 0.f;
+
+    for (int s = steps - 1; s >= 0; --s) {
+        float xp[VEC], xc[VEC], dv[VEC];
+        E::unpack(xl[s * kWave + lane], xp);
+        E::unpack(xl[s * kWave + lane + 1], xc);
+        E::unpack(dl[s * kWave + lane], dv);
+        // xw[i] = padded x at position (first position of the lane's vector) - (W-1) + i
+        float xw[VEC + W - 1], g[VEC + W - 1];
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i) xw[i] = xp[VEC - (W - 1) + i];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xw[W - 1 + e] = xc[e];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) g[e] = SILU ? __builtin_fmaf(dv[e], act_grad(&xw[e]), 0.f) : dv[e];
+#pragma unroll
+        for (int e = 0; e < W - 1; ++e) g[VEC + e] = from_next_lane(g[e], carry[e]);
+#pragma unroll
+        for (int e = 0; e < W - 1; ++e) carry[e] = read_lane(g[e], 0);
+        float dxv[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float acc = wv_[W - 1] * g[e];
+#pragma unroll
+            for (int k = 1; k < W; ++k) acc = fmaf(wv_[W - 1 - k], g[e + k], acc);
+            dxv[e] = acc;
+            dB += g[e];
+#pragma unroll
+            for (int k = 0; k < W; ++k) dW[k] = fmaf(g[e], xw[e + k], dW[k]);
+        }
+        const int p0 = (v0 + s * kWave + lane) * VEC;      // first position of the lane's vector
+        const int step_first = (v0 + s * kWave) * VEC;
+        if (has_dfinal && L - 1 >= step_first && L - (W - 1) < step_first + kWave * VEC) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+#pragma unroll
+                for (int i = 0; i < W - 1; ++i)
+                    if (p0 + e == L - (W - 1) + i) dxv[e] += dfin[i];
+        }
+        const u32x4 packed = E::pack(dxv);
+        // dwords behind the row's end are out of range: not stored
+        __builtin_amdgcn_raw_buffer_store_b128(packed, rdx, vd + s * 1024, 0, 2);
+        if (odd_tail && L - 1 >= p0 && L - 1 < p0 + VEC) {
+            T out[VEC];
+            __builtin_memcpy(out, &packed, sizeof(packed));
+            st_raw<DT>(dxrow, L - 1, out[(L - 1) - p0]);
+        }
+        // dinitial_states[i] is dx at position i - (W-1) in front of the row: the row's first lane
+        // has the g values it takes (csrc/causal_conv1d_bwd.cu:544-561)
+        if (a.dinitial_states != nullptr && tile == 0 && s == 0 && lane == 0) {
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) {
+                float acc = 0.f;
+#pragma unroll
+                for (int k = W - 1 - i; k < W; ++k) acc = fmaf(wv_[W - 1 - k], g[i - (W - 1) + k], acc);
+                st_elem<DT>(a.dinitial_states, (int64_t)b * a.dinit_stride_b + (int64_t)c * a.dinit_stride_c +
+                                                   (int64_t)i * a.dinit_stride_l, acc);
+            }
+        }
+    }
+
+    // The tile's sums over its lanes, in a fixed order, to plane (batch entry, tile) of the workspace.
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = wave_total_in_lane63(dW[w]);
+    dB = wave_total_in_lane63(dB);
+    if (lane == kWave - 1) {
+        float *dst = a.ws + ((int64_t)b * a.tiles_per_row + tile) * (int64_t)(W + 1) * a.dim + c;
+#pragma unroll
+        for (int w = 0; w < W; ++w) dst[(int64_t)w * a.dim] = dW[w];
+        dst[(int64_t)W * a.dim] = dB;
+    }
+}
+
+template <int DT, int W>
+int launch_tile_act(const cc1d_bwd_params &p, const BwdCfTileArgs &a, hipStream_t stream) {
+    const uint32_t blocks = (a.total + (kBlock / kWave) - 1) / (kBlock / kWave);
+    if (p.silu) CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, a);
+    else CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, a);
+    return launch_status();
+}
+
+template <int DT>
+int launch_tile_width(const cc1d_bwd_params &p, const BwdCfTileArgs &a, hipStream_t stream) {
+    switch (p.width) {
+        case 2: return launch_tile_act<DT, 2>(p, a, stream);
+        case 3: return launch_tile_act<DT, 3>(p, a, stream);
+        default: return launch_tile_act<DT, 4>(p, a, stream);
+    }
+}
+
+int64_t tiles_per_row(const cc1d_bwd_params &p) {
+    const int vec = vec_elems(p.x_dtype);
+    const int64_t n_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
+    return (n_vecs + kTileVecs - 1) / kTileVecs;
+}
+
+}  // namespace
+
+// Rows of more than 64 vectors (shorter ones share wavefronts in the short-row kernel), shorter
+// than 2 GiB; any alignment, any strides between rows.
+bool bwd_channelfirst_tile_applies(const cc1d_bwd_params &p) {
+    const int vec = vec_elems(p.x_dtype);
+    return ((int64_t)p.seqlen + vec - 1) / vec > kWave && (int64_t)p.seqlen * elem_bytes(p.x_dtype) < ((int64_t)1 << 31) - 64;
+}
+
+int bwd_channelfirst_tile_parts(const cc1d_bwd_params &p) { return (int)(p.batch * tiles_per_row(p)); }
+
+bool bwd_channelfirst_tile_fits(const cc1d_bwd_params &p) {
+    return (int64_t)p.batch * p.dim * tiles_per_row(p) < wave_limit() && (int64_t)p.batch * tiles_per_row(p) < ((int64_t)1 << 30);
+}
+
+int launch_bwd_channelfirst_tile(const cc1d_bwd_params &p, float *ws, hipStream_t stream) {
+    if (!bwd_channelfirst_tile_fits(p)) return CC1D_ERR_TOO_LARGE;
+    BwdCfTileArgs a = {};
+    a.tiles_per_row = (uint32_t)tiles_per_row(p);
+    a.total = (uint32_t)((int64_t)p.batch * p.dim * a.tiles_per_row);
+    a.seqlen = p.seqlen; a.batch = p.batch; a.dim = p.dim;
+    a.batch_inner = p.batch > 1 && p.dim > 1 && p.x_stride_b < p.x_stride_c ? 1 : 0;
+    a.w_dtype = p.w_dtype;
+    a.x = p.x; a.dout = p.dout; a.dx = p.dx; a.weight = p.weight; a.bias = p.bias; a.ws = ws;
+    a.x_stride_b = p.x_stride_b; a.x_stride_c = p.x_stride_c;
+    a.dout_stride_b = p.dout_stride_b; a.dout_stride_c = p.dout_stride_c;
+    a.dx_stride_b = p.dx_stride_b; a.dx_stride_c = p.dx_stride_c;
+    a.w_stride_c = p.w_stride_c; a.w_stride_w = p.w_stride_w;
+    a.initial_states = p.initial_states; a.dfinal_states = p.dfinal_states; a.dinitial_states = p.dinitial_states;
+    a.init_stride_b = p.init_stride_b; a.init_stride_c = p.init_stride_c; a.init_stride_l = p.init_stride_l;
+    a.dfinal_stride_b = p.dfinal_stride_b; a.dfinal_stride_c = p.dfinal_stride_c; a.dfinal_stride_l = p.dfinal_stride_l;
+    a.dinit_stride_b = p.dinit_stride_b; a.dinit_stride_c = p.dinit_stride_c; a.dinit_stride_l = p.dinit_stride_l;
+    switch (p.x_dtype) {
+        case CC1D_F32: return launch_tile_width<CC1D_F32>(p, a, stream);
+        case CC1D_F16: return launch_tile_width<CC1D_F16>(p, a, stream);
+        default: return launch_tile_width<CC1D_BF16>(p, a, stream);
+    }
+}
+
+}  // namespace cc1d

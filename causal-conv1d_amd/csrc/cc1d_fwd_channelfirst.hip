@@ -776,6 +776,9 @@ int launch_dtype(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t strea
 }  // namespace
 
 int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
+    // Rows of whole vectors on the 16-byte grid, longer than the short-row kernel takes: tile
+    // wavefronts (a forced segment length keeps such tensors on the walking kernels below).
+    if (tunables().fwd_cf_vecs == 0 && fwd_channelfirst_tile_applies(p)) return launch_fwd_channelfirst_tile(p, stream);
     const int vec = vec_elems(p.x_dtype);
     // The streaming kernel needs every row of out on the 16-byte grid of the same row of x;
     // steps per register set: two once a row has at least eight steps.

@@ -1,0 +1,211 @@
+// Channel-first forward for gfx950, rows of whole 16-byte vectors on the 16-byte grid (what a
+// contiguous (batch, dim, seqlen) tensor with seqlen a multiple of 8 (16-bit) or 4 (fp32) is):
+// short-lived tile wavefronts.  Takes over causal_conv1d_fwd_kernel
+// (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for these tensors; everything else stays
+// with the kernels of cc1d_fwd_channelfirst.hip.
+//
+// Design.  A wavefront takes a tile of up to four 64-vector steps (4 KiB) of one (batch, channel)
+// row and asks for all of it at once: the data goes from memory straight into LDS
+// (buffer_load_dwordx4 ... lds), together with the vector in front of the tile, whose last W-1
+// elements are the tile's halo.  No registers are held while the tile is in flight, a tile needs
+// 4.1 KB of LDS, and eight wavefronts fit a SIMD; they live for one memory round trip and a few
+// hundred instructions, so the launch moves through memory as one compact front in the order of
+// the rows instead of as thousands of long-lived streams.  The row is a buffer resource of its
+// own: the lane's vector is the vector offset, the step the instruction's immediate offset (which
+// the hardware adds to the LDS address as well), and what lies outside the row needs no test --
+// the vector in front of the first tile and the steps behind the row's end are out of range, read
+// as zeros and are not stored.  A lane's left neighbours come out of LDS (the upper half of the
+// previous vector), so there is no cross-lane traffic and no barrier.
+#include <type_traits>
+
+#include "cc1d_device.hpp"
+#include "cc1d_internal.hpp"
+
+namespace cc1d {
+namespace {
+
+constexpr int kTileSteps = 4;                     // 64-vector steps per tile
+constexpr int kTileVecs = kTileSteps * kWave;     // 256 vectors, 4 KiB
+constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
+
+typedef void __attribute__((address_space(3))) *lds_ptr_t;
+
+struct FwdCfTileArgs {
+    uint32_t total;               // rows * tiles_per_row wavefronts
+    uint32_t tiles_per_row;
+    int32_t n_vecs;               // vectors per row
+    int32_t batch, dim;
+    int32_t batch_inner;          // rows numbered with the batch entry fastest (see row_of)
+    int32_t w_dtype;
+    int32_t states;               // bit 0: initial_states given, bit 1: final_states wanted
+    const void *x;
+    void *out;
+    const void *weight;
+    const void *bias;
+    int64_t x_stride_b, x_stride_c, out_stride_b, out_stride_c;     // elements
+    int64_t w_stride_c, w_stride_w;
+    const void *initial_states;
+    void *final_states;
+    int64_t init_stride_b, init_stride_c, init_stride_l;
+    int64_t final_stride_b, final_stride_c, final_stride_l;
+};
+
+template <int DT, int W, bool SILU>
+__global__ void __launch_bounds__(kBlock, 4)
+fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
+    using E = Elem<DT>;
+    using T = typename E::type;
+    constexpr int VEC = E::kVec;
+    constexpr bool PRECISE = E::kPreciseAct;
+    constexpr bool SCALED = SILU && !PRECISE;         // taps and bias carry the factor of the SiLU exponent
+    __shared__ u32x4 lds[kBlock / kWave][kTileVecs + 1];   // [wavefront][halo vector + tile]
+
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
+    const int lane = (int)(threadIdx.x & (kWave - 1));
+    const uint32_t wid = blockIdx.x * (uint32_t)(kBlock / kWave) + (uint32_t)wv;
+    if (wid >= a.total) return;
+    const int tile = (int)(wid % a.tiles_per_row);
+    const uint32_t row = wid / a.tiles_per_row;
+    // Channels run fastest for tensors whose rows lie in (batch, dim) order in memory; for a
+    // (dim, batch, seqlen) tensor seen as (batch, dim, seqlen) the batch entries of a channel are
+    // the neighbours in memory and run fastest instead.
+    int b, c;
+    if (a.batch_inner) { b = (int)(row % (uint32_t)a.batch); c = (int)(row / (uint32_t)a.batch); }
+    else { c = (int)(row % (uint32_t)a.dim); b = (int)(row / (uint32_t)a.dim); }
+
+    const T *xrow = reinterpret_cast<const T *>(a.x) + (int64_t)b * a.x_stride_b + (int64_t)c * a.x_stride_c;
+    T *orow = reinterpret_cast<T *>(a.out) + (int64_t)b * a.out_stride_b + (int64_t)c * a.out_stride_c;
+    const int row_bytes = a.n_vecs * 16;
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xrow), 0, row_bytes, kRsrcRaw);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(orow, 0, row_bytes, kRsrcRaw);
+    const int v0 = tile * kTileVecs;                  // the tile's first vector
+    int steps = (a.n_vecs - v0 + kWave - 1) / kWave;  // steps of the tile that reach into the row
+    steps = steps > kTileSteps ? kTileSteps : steps;
+    // LDS vector i of the wavefront holds row vector v0 - 1 + i.  For the row's first tile the
+    // offset below wraps around: out of range, LDS gets zeros (the row's zero padding).
+    const int vx = (lane + v0 - 1) * 16;
+    u32x4 *mine = &lds[wv][0];
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 0, 2);
+    if (steps > 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 1024, 2);
+    if (steps > 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 2048, 2);
+    if (steps > 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 3072, 2);
+    if (lane == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(mine + steps * kWave), 16, vx + steps * 1024, 0, 0, 2);
+
+    float wv_[W], bias_v;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+        wv_[w] = ld_weight(a.weight, a.w_dtype, (int64_t)c * a.w_stride_c + w * a.w_stride_w);
+    bias_v = a.bias == nullptr ? 0.f : ld_weight(a.bias, a.w_dtype, c);
+    if (SCALED) {
+        bias_v *= kSiluPrescale;
+#pragma unroll
+        for (int w = 0; w < W; ++w) wv_[w] *= kSiluPrescale;
+    }
+    // The row's first tile takes initial_states as its halo: its first lane fetches the W-1 values.
+    float init[W - 1];
+#pragma unroll
+    for (int i = 0; i < W - 1; ++i) init[i] = 0.f;
+    const bool first_lane_of_row = tile == 0 && lane == 0;
+    if ((a.states & 1) != 0 && first_lane_of_row) {
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i)
+            init[i] = ld_elem<DT>(a.initial_states, (int64_t)b * a.init_stride_b + (int64_t)c * a.init_stride_c +
+                                                        (int64_t)i * a.init_stride_l);
+    }
+    // Every vector of the tile is in LDS behind this wait (a vector fetched into LDS counts as a
+    // load until it has been written there).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    for (int s = 0; s < steps; ++s) {
+        float xp[VEC], xc[VEC];
+        E::unpack(mine[s * kWave + lane], xp);
+        E::unpack(mine[s * kWave + lane + 1], xc);
+        // xx[i] = padded x at position (first position of the lane's vector) - (W-1) + i
+        float xx[VEC + W - 1];
+#pragma unroll
+        for (int i = 0; i < W - 1; ++i) xx[i] = xp[VEC - (W - 1) + i];
+        if (s == 0 && first_lane_of_row) {
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) xx[i] = init[i];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xx[W - 1 + e] = xc[e];
+        float acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float s_ = bias_v;
+#pragma unroll
+            for (int w = 0; w < W; ++w) s_ = fmaf(wv_[w], xx[e + w], s_);
+            acc[e] = SCALED ? silu_from_scaled(s_) : SILU ? silu<PRECISE>(s_) : s_;
+        }
+        // vectors behind the row's end are out of range: not stored
+        __builtin_amdgcn_raw_buffer_store_b128(E::pack(acc), ro, (lane + v0) * 16 + s * 1024, 0, 2);
+    }
+
+    // final_states[b, c, i] = x[L-(W-1)+i], copied by the wavefront of the row's FIRST tile, the
+    // one that read initial_states: the two may be one buffer, and inside one wavefront the
+    // reads are complete (the wait above) before the stores.  Rows here hold more than 64
+    // vectors, so the values all come from x.
+    if ((a.states & 2) != 0 && tile == 0 && lane < W - 1) {
+        const int L = a.n_vecs * VEC;
+        const T v = ld_raw<DT>(xrow, L - (W - 1) + lane);
+        st_raw<DT>(a.final_states, (int64_t)b * a.final_stride_b + (int64_t)c * a.final_stride_c +
+                                       (int64_t)lane * a.final_stride_l, v);
+    }
+}
+
+template <int DT, int W>
+int launch_tile_act(const cc1d_fwd_params &p, const FwdCfTileArgs &a, hipStream_t stream) {
+    const uint32_t blocks = (a.total + (kBlock / kWave) - 1) / (kBlock / kWave);
+    if (p.silu) CC1D_LAUNCH((fwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, a);
+    else CC1D_LAUNCH((fwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, a);
+    return launch_status();
+}
+
+template <int DT>
+int launch_tile_width(const cc1d_fwd_params &p, const FwdCfTileArgs &a, hipStream_t stream) {
+    switch (p.width) {
+        case 2: return launch_tile_act<DT, 2>(p, a, stream);
+        case 3: return launch_tile_act<DT, 3>(p, a, stream);
+        default: return launch_tile_act<DT, 4>(p, a, stream);
+    }
+}
+
+}  // namespace
+
+// Rows of whole vectors, every row of x and of out starting on the 16-byte grid, more vectors
+// per row than the short-row kernel takes, and a row shorter than 2 GiB.
+bool fwd_channelfirst_tile_applies(const cc1d_fwd_params &p) {
+    const int vec = vec_elems(p.x_dtype);
+    return p.seqlen % vec == 0 && p.seqlen / vec > kWave && (int64_t)p.seqlen * elem_bytes(p.x_dtype) < ((int64_t)1 << 31) &&
+           aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
+           aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
+}
+
+int launch_fwd_channelfirst_tile(const cc1d_fwd_params &p, hipStream_t stream) {
+    const int vec = vec_elems(p.x_dtype);
+    FwdCfTileArgs a = {};
+    a.n_vecs = p.seqlen / vec;
+    a.tiles_per_row = (uint32_t)((a.n_vecs + kTileVecs - 1) / kTileVecs);
+    const int64_t total = (int64_t)p.batch * p.dim * a.tiles_per_row;
+    if (total >= wave_limit()) return CC1D_ERR_TOO_LARGE;
+    a.total = (uint32_t)total;
+    a.batch = p.batch; a.dim = p.dim;
+    a.batch_inner = p.batch > 1 && p.dim > 1 && p.x_stride_b < p.x_stride_c ? 1 : 0;
+    a.w_dtype = p.w_dtype;
+    a.states = (p.initial_states != nullptr ? 1 : 0) | (p.final_states != nullptr ? 2 : 0);
+    a.x = p.x; a.out = p.out; a.weight = p.weight; a.bias = p.bias;
+    a.x_stride_b = p.x_stride_b; a.x_stride_c = p.x_stride_c;
+    a.out_stride_b = p.out_stride_b; a.out_stride_c = p.out_stride_c;
+    a.w_stride_c = p.w_stride_c; a.w_stride_w = p.w_stride_w;
+    a.initial_states = p.initial_states; a.final_states = p.final_states;
+    a.init_stride_b = p.init_stride_b; a.init_stride_c = p.init_stride_c; a.init_stride_l = p.init_stride_l;
+    a.final_stride_b = p.final_stride_b; a.final_stride_c = p.final_stride_c; a.final_stride_l = p.final_stride_l;
+    switch (p.x_dtype) {
+        case CC1D_F32: return launch_tile_width<CC1D_F32>(p, a, stream);
+        case CC1D_F16: return launch_tile_width<CC1D_F16>(p, a, stream);
+        default: return launch_tile_width<CC1D_BF16>(p, a, stream);
+    }
+}
+
+}  // namespace cc1d

@@ -101,12 +101,21 @@ inline int launch_status() {
 
 int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *gather, hipStream_t stream);
 int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream);
+// Channel-first rows of whole vectors on the 16-byte grid: the tile kernel (cc1d_fwd_channelfirst_tile.hip).
+bool fwd_channelfirst_tile_applies(const cc1d_fwd_params &p);
+int launch_fwd_channelfirst_tile(const cc1d_fwd_params &p, hipStream_t stream);
 
 size_t bwd_channellast_workspace_bytes(const cc1d_bwd_params &p);
 size_t bwd_channelfirst_workspace_bytes(const cc1d_bwd_params &p);
 // false: the launcher would answer CC1D_ERR_TOO_LARGE (and launch nothing).
 bool bwd_channellast_fits(const cc1d_bwd_params &p);
 bool bwd_channelfirst_fits(const cc1d_bwd_params &p);
+// Channel-first rows of more than 64 vectors: the tile kernel (cc1d_bwd_channelfirst_tile.hip);
+// its workspace is `parts` planes of (width + 1) x dim floats.
+bool bwd_channelfirst_tile_applies(const cc1d_bwd_params &p);
+bool bwd_channelfirst_tile_fits(const cc1d_bwd_params &p);
+int bwd_channelfirst_tile_parts(const cc1d_bwd_params &p);
+int launch_bwd_channelfirst_tile(const cc1d_bwd_params &p, float *ws, hipStream_t stream);
 int launch_bwd_channellast(const cc1d_bwd_params &p, void *ws, hipStream_t stream);
 int launch_bwd_channelfirst(const cc1d_bwd_params &p, void *ws, hipStream_t stream);
 // Second stage of both backward layouts: ordered sum of the workspace planes into dweight/dbias.

@@ -79,9 +79,10 @@ def test_no_alloc_backward_equals_backward_with_workspace(gpu_device, cc1d_lib, 
 
 @pytest.mark.gpu
 def test_no_alloc_backward_without_workspace_need(gpu_device, cc1d_lib):
-    """Channel-first with 4096 channels and more is one part per channel: no workspace at all."""
+    """Channel-first rows of at most 64 vectors with 4096 channels and more are one part per
+    channel: no workspace at all."""
     lib = cabi.declare(cc1d_lib)
-    host, d = _problem(1, 4096, 520, torch.bfloat16, False, 510, gpu_device)
+    host, d = _problem(1, 4096, 504, torch.bfloat16, False, 510, gpu_device)
     ref, need = _run(lib, d, gpu_device, noalloc=False)
     got, _ = _run(lib, d, gpu_device, noalloc=True)
     assert need == 0
