@@ -1,8 +1,9 @@
-// Channel-first forward for gfx950, rows of whole 16-byte vectors on the 16-byte grid (what a
-// contiguous (batch, dim, seqlen) tensor with seqlen a multiple of 8 (16-bit) or 4 (fp32) is):
-// short-lived tile wavefronts.  Takes over causal_conv1d_fwd_kernel
-// (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for these tensors; everything else stays
-// with the kernels of cc1d_fwd_channelfirst.hip.
+// Channel-first forward for gfx950, rows of 65 to 128 whole 16-byte vectors on the 16-byte grid
+// (a contiguous (batch, dim, seqlen) tensor with seqlen 520 .. 1024 in 16-bit data, a multiple of
+// 8; 260 .. 512 in fp32, a multiple of 4): short-lived tile wavefronts.  Takes over
+// causal_conv1d_fwd_kernel (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for these tensors;
+// everything else stays with the kernels of cc1d_fwd_channelfirst.hip (see
+// fwd_channelfirst_tile_applies below for the measurements behind the limits).
 //
 // Design.  A wavefront takes a tile of up to four 64-vector steps (4 KiB) of one (batch, channel)
 // row and asks for all of it at once: the data goes from memory straight into LDS
@@ -35,7 +36,7 @@ struct FwdCfTileArgs {
     uint32_t tiles_per_row;
     int32_t n_vecs;               // vectors per row
     int32_t batch, dim;
-    int32_t batch_inner;          // rows numbered with the batch entry fastest (see row_of)
+    int32_t batch_inner;          // rows numbered with the batch entry fastest
     int32_t w_dtype;
     int32_t states;               // bit 0: initial_states given, bit 1: final_states wanted
     const void *x;
@@ -174,10 +175,17 @@ int launch_tile_width(const cc1d_fwd_params &p, const FwdCfTileArgs &a, hipStrea
 }  // namespace
 
 // Rows of whole vectors, every row of x and of out starting on the 16-byte grid, more vectors
-// per row than the short-row kernel takes, and a row shorter than 2 GiB.
+// per row than the short-row kernel takes (64) and at most twice as many: there a walking
+// wavefront has one or two steps and nothing to overlap its own latency with, and tiles measured
+// 8-15 % faster ((4, 5376, 520) bf16 15.2 -> 13.1 us, (4, 5376, 768) 15.9 -> 13.8, (16, 5376, 1024)
+// 60.7 -> 55.8, (64, 2048, 1024) fp16 with states 105.7 -> 89.5 us).  Longer rows keep the walking
+// kernel, whose 256-vector segments are short-lived wavefronts already and which holds its rows in
+// registers: tiles measured 2-6 % slower there ((4, 2048, 4096) bf16 23.3 -> 23.6 us, (8, 5376, 2048)
+// 57.1 -> 59.9 us) and 16 % slower on rows that do not end on cache lines ((8, 5376, 2000) 56.5 -> 65.5 us).
 bool fwd_channelfirst_tile_applies(const cc1d_fwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
-    return p.seqlen % vec == 0 && p.seqlen / vec > kWave && (int64_t)p.seqlen * elem_bytes(p.x_dtype) < ((int64_t)1 << 31) &&
+    return p.seqlen % vec == 0 && p.seqlen / vec > kWave && p.seqlen / vec <= 2 * kWave &&
+           (int64_t)p.seqlen * elem_bytes(p.x_dtype) < ((int64_t)1 << 31) &&
            aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
            aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
 }
