@@ -17,8 +17,9 @@ Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill 
                      back-to-back launches of the same call, so the clock has settled where it
                      stays under load; `frac_burst` is the same K steps out of an idle device
                      (a few milliseconds of load at the highest clock); `frac_rotated` runs over
-                     six rotating sets of x and out (2.1 GB), where every launch meets cold caches
-                     and address translations, as the layers of a model do.  `decode` repeats
+                     six rotating sets of x and out (2.1 GB), where no launch finds its tensors in
+                     a cache, as the layers of a model do, behind the same 400 untimed launches
+                     (none with --no-settle).  `decode` repeats
                      the three figures for the two decode-step updates.  `traffic` is imported
                      from the committed rocprofv3 summary, not measured in this run
   cpu_baseline ..... the PyTorch oracle (F.conv1d per packed sub-sequence) timed on this
@@ -415,7 +416,8 @@ def main():
                     help="launches timed per decode-step figure (at least --steps); counter passes use few")
     ap.add_argument("--only", choices=["update", "rotated"], default=None,
                     help="update: time nothing but the warm decode-step launches (linear, then circular); "
-                         "rotated: nothing but the headline forward over its six rotating buffer sets.  The "
+                         "rotated: nothing but the headline forward over its six rotating buffer sets, then "
+                         "torch.add over the same sets (K steps each behind --warmup untimed ones).  The "
                          "commands whose rocprofv3 kernel traces and counters give device durations and traffic")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain device copy of x (a kernel of known size, to scale profiler counters)")
@@ -452,9 +454,11 @@ def main():
         sets = rotated_sets()
         rot_us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(sets[i % 6][0], w, b, seq, None, sets[i % 6][1], None, True),
                              args.steps, args.warmup)
+        add_us, _ = time_gpu(lambda i: torch.add(sets[i % 6][0], 1.0, out=sets[i % 6][1]), args.steps, args.warmup)
         print(json.dumps({"only": "rotated", "steps": args.steps, "warmup": args.warmup, "rotated_sets": 6,
                           "us_per_call_rotated": round(rot_us, 3), "algorithmic_bytes": int(n_bytes),
-                          "frac_rotated": round(gbs(n_bytes, rot_us) / HBM_PEAK_GBS, 4)}), flush=True)
+                          "frac_rotated": round(gbs(n_bytes, rot_us) / HBM_PEAK_GBS, 4),
+                          "us_torch_add_rotated": round(add_us, 3)}), flush=True)
         return
 
     # The burst: K steps out of an idle device.  Then the figure the line carries: the same K steps
@@ -514,13 +518,13 @@ def main():
         line["roofline"]["traffic_source"] = {"profile": prof["profile"], "imported": True,
                                               "kernel_sources_sha16": prof["kernel_sources_sha16"]}
     if not args.no_others and not args.no_rotated:
-        # The same call over six rotating sets of x and out (2.1 GB): every launch then meets cold
-        # address translations and caches, as the layers of a model do; next to it PyTorch's
-        # elementwise add over the same sets (the same bytes in, the same bytes out).
+        # The same call over six rotating sets of x and out (2.1 GB): no launch finds its tensors in a
+        # cache, as the layers of a model do; next to it PyTorch's elementwise add over the same sets
+        # (the same bytes in, the same bytes out).  Both behind the same untimed launches as `value`.
         sets = rotated_sets()
         rot_us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(sets[i % 6][0], w, b, seq, None, sets[i % 6][1], None, True),
-                             args.steps, args.warmup)
-        add_us, _ = time_gpu(lambda i: torch.add(sets[i % 6][0], 1.0, out=sets[i % 6][1]), args.steps, args.warmup)
+                             args.steps, args.warmup + settle)
+        add_us, _ = time_gpu(lambda i: torch.add(sets[i % 6][0], 1.0, out=sets[i % 6][1]), args.steps, args.warmup + settle)
         line["config"].update({"us_per_call_rotated": round(rot_us, 3), "rotated_sets": 6,
                                "GBps_rotated": round(gbs(n_bytes, rot_us), 1),
                                "us_torch_add_rotated": round(add_us, 3)})

@@ -30,6 +30,12 @@
 // rows longer than 64 vectors.  The short-row kernel takes rows of at most 64 vectors (whole
 // vectors on one grid, or element by element), several batch entries of a channel to a
 // wavefront and no walk.
+//
+// Rows longer than 64 vectors normally do not reach these walking kernels: the tile kernel of
+// cc1d_bwd_channelfirst_tile.hip takes them (a wavefront per tile of up to 256 vectors of one
+// row, fetched straight into LDS; one workspace plane per tile and the shared second stage), at
+// any length and alignment.  The launch tunable bwd_cf_parts = -1 brings the walking kernels
+// back for the same tensors; dx and dinitial_states are bit-identical either way.
 #include <type_traits>
 
 #include "cc1d_device.hpp"

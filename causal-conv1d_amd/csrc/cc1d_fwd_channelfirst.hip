@@ -26,7 +26,10 @@
 // the few positions of a row in front of its first whole vector or behind its last one are
 // produced one per lane, straight from memory.  The general kernel takes out tensors on a different grid.  The short-row
 // kernel takes rows of at most 64 vectors, several rows to a wavefront and no walk; the flat
-// kernel takes such rows of a contiguous tensor as whole vectors of one flat array.
+// kernel takes such rows of a contiguous tensor as whole vectors of one flat array.  Rows of
+// 65 to 128 whole vectors on the 16-byte grid go to the tile kernel of
+// cc1d_fwd_channelfirst_tile.hip (rows fetched straight into LDS; 8-15 % faster there, slower
+// than the walk for longer rows); the launch tunable fwd_cf_vecs = -1 keeps them here.
 #include <type_traits>
 
 #include "cc1d_device.hpp"

@@ -118,7 +118,9 @@ int cc1d_fwd(const cc1d_fwd_params *p, cc1d_stream_t stream);
  *
  * The workspace is caller-owned device memory, 16-byte aligned, of at least
  * cc1d_bwd_workspace_bytes() bytes (the reference allocates its own with at::zeros,
- * causal_conv1d.cpp:396-429).  It needs no initialisation.
+ * causal_conv1d.cpp:396-429).  It needs no initialisation.  A problem too large for one grid is
+ * launched as slices of the batch, one after the other on the stream, each adding into
+ * dweight / dbias: the sums then follow the slice order (still the same bits run to run).
  * ---------------------------------------------------------------------------------- */
 typedef struct cc1d_bwd_params {
     int32_t batch, dim, seqlen, width;
@@ -163,8 +165,10 @@ int cc1d_bwd(const cc1d_bwd_params *p, void *workspace, size_t workspace_bytes,
  * (one copy per GPU, held from the first use of the library on that GPU until the process ends).
  * A problem whose cc1d_bwd_workspace_bytes() exceeds that size is refused with
  * CC1D_ERR_WORKSPACE_LIMIT before anything is launched (16 MiB covers, for instance, the bf16
- * prefill shape (8, 5376, 2048) channel-last at 13.8 MB; channel-first problems with dim >= 4096
- * need none).  Calls no hipMalloc / hipFree and nothing that allocates.  The device that owns
+ * prefill shape (8, 5376, 2048) channel-last at 13.8 MB; a channel-first problem needs
+ * batch x ceil(row vectors / 256) x (width + 1) x dim floats once its rows are longer than 64
+ * sixteen-byte vectors -- 1.3 MB for fp16 (4, 4096, 8192) -- and none for shorter rows at
+ * dim >= 4096).  Calls no hipMalloc / hipFree and nothing that allocates.  The device that owns
  * `stream` must be the current device.  All calls on one GPU share that GPU's array: calls that
  * overlap in time on one GPU (different streams, no ordering between them) race; calls on one
  * stream never do.  The array needs no clearing between calls (every plane that is read was
