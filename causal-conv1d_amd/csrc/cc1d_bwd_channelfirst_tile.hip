@@ -23,7 +23,10 @@
 // where the walking kernel took 2.2 times as long), and what lies outside a row needs no test:
 // the vector in front of the first tile and everything behind the row's end is out of range,
 // reads as zero and is not stored.  A 16-bit row of odd length ends in half a dword, which the
-// range check would drop: that one element is fetched and stored on its own.
+// range check would drop: that one element is fetched and stored on its own.  A row whose last
+// 64-vector step would hold at most 64 positions ends in a tail instead: the row's last tile
+// fetches those vectors as well and takes their positions one per lane, ahead of its steps
+// ((16, 4096, 1025) bf16 103 -> 87 us, 2049: 194 -> 149 us; 1024 / 2048: 77 / 134 us).
 // The steps of a tile are computed top down.  A lane's x halo is the upper half of the previous
 // vector in LDS; the g values to the right of its vector come from the next lane (DPP shift),
 // for the last lane from the step above (carried), for the top step from the vectors behind the
@@ -41,6 +44,7 @@ namespace {
 
 constexpr int kTileSteps = 4;                     // 64-vector steps per tile
 constexpr int kTileVecs = kTileSteps * kWave;     // 256 vectors, 4 KiB per tensor
+constexpr int kTailVecs = kWave / 4;              // most vectors 64 positions can span (fp32)
 constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
 
 typedef void __attribute__((address_space(3))) *lds_ptr_t;
@@ -49,6 +53,8 @@ struct BwdCfTileArgs {
     uint32_t total;               // rows * tiles_per_row wavefronts
     uint32_t tiles_per_row;
     int32_t seqlen;
+    int32_t body_vecs;            // vectors of a row that are walked as vectors (all of them, or a whole number of steps)
+    int32_t tail_vecs;            // vectors behind them, done one position per lane (0: none)
     int32_t batch, dim;
     int32_t batch_inner;          // rows numbered with the batch entry fastest
     int32_t w_dtype;
@@ -88,7 +94,7 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     constexpr int VEC = E::kVec;
     constexpr int EB = E::kBytes;
     constexpr bool PRECISE = E::kPreciseAct;
-    constexpr int XV = kTileVecs + 2, DV = kTileVecs + 1;     // vectors of x and of dout a tile holds
+    constexpr int XV = kTileVecs + 2 + kTailVecs, DV = kTileVecs + 1 + kTailVecs;   // vectors of x and of dout a tile holds
     __shared__ u32x4 lds[kBlock / kWave][XV + DV];
 
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
@@ -112,10 +118,13 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xrow), 0, row_bytes, kRsrcRaw);
     const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(drow), 0, row_bytes, kRsrcRaw);
     const __amdgpu_buffer_rsrc_t rdx = __builtin_amdgcn_make_buffer_rsrc(dxrow, 0, row_bytes, kRsrcRaw);
-    const int n_vecs = (L + VEC - 1) / VEC;
     const int v0 = tile * kTileVecs;                  // the tile's first vector
-    int steps = (n_vecs - v0 + kWave - 1) / kWave;    // steps of the tile that reach into the row
+    int steps = (a.body_vecs - v0 + kWave - 1) / kWave;   // steps of the tile that reach into the row
     steps = steps > kTileSteps ? kTileSteps : steps;
+    // A row whose last step would hold at most 64 positions ends in a tail instead: its last tile
+    // fetches those vectors too and takes their positions one per lane (an eighth of a step's
+    // instructions instead of a whole step for a handful of lanes).
+    const int tail_vecs = tile == (int)a.tiles_per_row - 1 ? a.tail_vecs : 0;
     // x vector i of the wavefront's LDS holds row vector v0 - 1 + i, dout vector i holds v0 + i.
     // For the row's first tile the x offset below wraps around: out of range, zeros.
     u32x4 *xl = &lds[wv][0], *dl = &lds[wv][XV];
@@ -134,9 +143,10 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 3072, 2);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 3072, 2);
     }
-    // behind the tile: two more vectors of x, one of dout (what the top step's last lane needs)
-    if (lane < 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(xl + steps * kWave), 16, vx + steps * 1024, 0, 0, 0);
-    if (lane < 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)(dl + steps * kWave), 16, vd + steps * 1024, 0, 0, 0);
+    // behind the tile: two more vectors of x, one of dout (what the top step's last lane needs),
+    // and the row's tail
+    if (lane < 2 + tail_vecs) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(xl + steps * kWave), 16, vx + steps * 1024, 0, 0, 0);
+    if (lane < 1 + tail_vecs) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)(dl + steps * kWave), 16, vd + steps * 1024, 0, 0, 0);
 
     // Taps and bias of the channel (wave-uniform); with the fast activation also times -log2(e),
     // so that the sum over the window is the exponent the derivative needs.
@@ -151,7 +161,7 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
 
     // What the resources leave out, fetched by single lanes: the odd last element of a 16-bit row
     // (by the tile that holds it) and initial_states in front of the row (by its first tile).
-    const int tile_first = v0 * VEC, tile_end = (v0 + steps * kWave) * VEC;     // positions [tile_first, tile_end)
+    const int tile_first = v0 * VEC, tile_end = (v0 + steps * kWave + tail_vecs) * VEC;   // positions [tile_first, tile_end)
     const bool holds_last = odd_tail && L - 1 >= tile_first - VEC && L - 1 < tile_end + VEC;
     T last_x = T(0.f), last_d = T(0.f);
     if (holds_last && lane == 0) {
@@ -191,11 +201,43 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) reinterpret_cast<T *>(xl)[VEC - (W - 1) + i] = init_raw[i];
     }
+    asm volatile("" ::: "memory");                    // the elements written above are read below as parts of vectors
 
     auto act_grad = [&](const float *xwin) { return silu_grad_of_window<W, PRECISE>(wv_, bias_v, wvs, bias_s, xwin); };
-    // g at the W-1 positions behind the tile, by every lane (the values are wave-uniform)
+    float dW[W], dB = 0.f;
+#pragma unroll
+    for (int w = 0; w < W; ++w) dW[w] = 0.f;
+    // g at the W-1 positions behind the tile's steps, in every lane (the values are wave-uniform)
     float carry[W - 1];
-    {
+    if (tail_vecs > 0) {
+        // The row's tail, one position per lane; lanes behind the row's end hold zeros.  Every lane
+        // takes part in the lane shifts.
+        const int p = (v0 + steps * kWave) * VEC + lane;
+        const bool in_row = p < L;
+        const T *xe = reinterpret_cast<const T *>(xl) + (p + VEC - tile_first) - (W - 1);
+        float xw[W];
+#pragma unroll
+        for (int k = 0; k < W; ++k) xw[k] = in_row ? E::to_float(xe[k]) : 0.f;
+        const float dv = in_row ? E::to_float(reinterpret_cast<const T *>(dl)[p - tile_first]) : 0.f;
+        float g[W];
+        g[0] = SILU ? __builtin_fmaf(dv, act_grad(xw), 0.f) : dv;
+#pragma unroll
+        for (int k = 1; k < W; ++k) g[k] = from_next_lane(g[k - 1], 0.f);
+        float acc = wv_[W - 1] * g[0];
+#pragma unroll
+        for (int k = 1; k < W; ++k) acc = fmaf(wv_[W - 1 - k], g[k], acc);
+        if (has_dfinal) {
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i)
+                if (p == L - (W - 1) + i) acc += dfin[i];
+        }
+        if (in_row) st_elem<DT>(dxrow, p, acc);
+        dB += g[0];
+#pragma unroll
+        for (int k = 0; k < W; ++k) dW[k] = fmaf(g[0], xw[k], dW[k]);
+#pragma unroll
+        for (int e = 0; e < W - 1; ++e) carry[e] = read_lane(g[0], e);
+    } else {
         float xa[VEC], xb[VEC], dv[VEC];
         E::unpack(xl[steps * kWave], xa);
         E::unpack(xl[steps * kWave + 1], xb);
@@ -206,9 +248,6 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
 #pragma unroll
         for (int e = 0; e < W - 1; ++e) carry[e] = SILU ? __builtin_fmaf(dv[e], act_grad(&xwin[e]), 0.f) : dv[e];
     }
-    float dW[W], dB = 0.f;
-#pragma unroll
-    for (int w = 0; w < W; ++w) dW[w] = 0.f;
 
     for (int s = steps - 1; s >= 0; --s) {
         float xp[VEC], xc[VEC], dv[VEC];
@@ -298,10 +337,17 @@ int launch_tile_width(const cc1d_bwd_params &p, const BwdCfTileArgs &a, hipStrea
     }
 }
 
+// The vectors of a row's last, partly filled step when they hold at most 64 positions.
+int tail_vecs_of_row(const cc1d_bwd_params &p) {
+    const int vec = vec_elems(p.x_dtype);
+    const int rem = (int)((((int64_t)p.seqlen + vec - 1) / vec) % kWave);
+    return rem > 0 && rem * vec <= kWave ? rem : 0;
+}
+
 int64_t tiles_per_row(const cc1d_bwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
-    const int64_t n_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
-    return (n_vecs + kTileVecs - 1) / kTileVecs;
+    const int64_t body_vecs = ((int64_t)p.seqlen + vec - 1) / vec - tail_vecs_of_row(p);
+    return (body_vecs + kTileVecs - 1) / kTileVecs;
 }
 
 }  // namespace
@@ -325,6 +371,8 @@ int launch_bwd_channelfirst_tile(const cc1d_bwd_params &p, float *ws, hipStream_
     a.tiles_per_row = (uint32_t)tiles_per_row(p);
     a.total = (uint32_t)((int64_t)p.batch * p.dim * a.tiles_per_row);
     a.seqlen = p.seqlen; a.batch = p.batch; a.dim = p.dim;
+    a.tail_vecs = tail_vecs_of_row(p);
+    a.body_vecs = (int32_t)(((int64_t)p.seqlen + vec_elems(p.x_dtype) - 1) / vec_elems(p.x_dtype)) - a.tail_vecs;
     a.batch_inner = p.batch > 1 && p.dim > 1 && p.x_stride_b < p.x_stride_c ? 1 : 0;
     a.w_dtype = p.w_dtype;
     a.x = p.x; a.dout = p.dout; a.dx = p.dx; a.weight = p.weight; a.bias = p.bias; a.ws = ws;

@@ -27,9 +27,10 @@
 // produced one per lane, straight from memory.  The general kernel takes out tensors on a different grid.  The short-row
 // kernel takes rows of at most 64 vectors, several rows to a wavefront and no walk; the flat
 // kernel takes such rows of a contiguous tensor as whole vectors of one flat array.  Rows of
-// 65 to 128 whole vectors on the 16-byte grid go to the tile kernel of
-// cc1d_fwd_channelfirst_tile.hip (rows fetched straight into LDS; 8-15 % faster there, slower
-// than the walk for longer rows); the launch tunable fwd_cf_vecs = -1 keeps them here.
+// 65 to 128 whole vectors on the 16-byte grid, and rows off that grid of up to 512 vectors (192
+// of fp32), go to the tile kernel of cc1d_fwd_channelfirst_tile.hip (rows fetched straight into
+// LDS; 8-15 % faster on the grid, 10-40 % off it, slower than the walk for longer rows); the
+// launch tunable fwd_cf_vecs = -1 keeps them here.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -779,8 +780,8 @@ int launch_dtype(const cc1d_fwd_params &p, const FwdCfGeom &g, hipStream_t strea
 }  // namespace
 
 int launch_fwd_channelfirst(const cc1d_fwd_params &p, hipStream_t stream) {
-    // Rows of whole vectors on the 16-byte grid, longer than the short-row kernel takes: tile
-    // wavefronts (a forced segment length keeps such tensors on the walking kernels below).
+    // Rows a little longer than the short-row kernel takes, and longer rows off the 16-byte grid:
+    // tile wavefronts (a forced segment length keeps such tensors on the walking kernels below).
     if (tunables().fwd_cf_vecs == 0 && fwd_channelfirst_tile_applies(p)) return launch_fwd_channelfirst_tile(p, stream);
     const int vec = vec_elems(p.x_dtype);
     // The streaming kernel needs every row of out on the 16-byte grid of the same row of x;

@@ -1,9 +1,11 @@
-// Channel-first forward for gfx950, rows of 65 to 128 whole 16-byte vectors on the 16-byte grid
-// (a contiguous (batch, dim, seqlen) tensor with seqlen 520 .. 1024 in 16-bit data, a multiple of
-// 8; 260 .. 512 in fp32, a multiple of 4): short-lived tile wavefronts.  Takes over
-// causal_conv1d_fwd_kernel (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for these tensors;
-// everything else stays with the kernels of cc1d_fwd_channelfirst.hip (see
-// fwd_channelfirst_tile_applies below for the measurements behind the limits).
+// Channel-first forward for gfx950: short-lived tile wavefronts.  Takes over
+// causal_conv1d_fwd_kernel (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for rows of 65 to
+// 128 whole 16-byte vectors on the 16-byte grid (a contiguous (batch, dim, seqlen) tensor with
+// seqlen 520 .. 1024 in 16-bit data, 260 .. 512 in fp32) and for rows off that grid -- a length
+// that is no whole number of vectors, a view that starts inside a vector, out on another grid
+// than x -- of up to 512 vectors of 16-bit data, 192 of fp32.  Everything else stays with the
+// kernels of cc1d_fwd_channelfirst.hip (see fwd_channelfirst_tile_applies below for the
+// measurements behind the limits).
 //
 // Design.  A wavefront takes a tile of up to four 64-vector steps (4 KiB) of one (batch, channel)
 // row and asks for all of it at once: the data goes from memory straight into LDS
@@ -16,7 +18,12 @@
 // the hardware adds to the LDS address as well), and what lies outside the row needs no test --
 // the vector in front of the first tile and the steps behind the row's end are out of range, read
 // as zeros and are not stored.  A lane's left neighbours come out of LDS (the upper half of the
-// previous vector), so there is no cross-lane traffic and no barrier.
+// previous vector), so there is no cross-lane traffic and no barrier.  The resource is based at
+// the row's first element wherever that lies (vector accesses need no alignment), so rows of any
+// length anywhere in memory take the same path; a 16-bit row of odd length ends in half a dword,
+// which the range check would drop: that one element is fetched and stored on its own.  A row
+// whose last 64-vector step would hold at most 64 positions ends in a tail instead: the last
+// tile fetches those vectors as well and produces their positions one per lane.
 #include <type_traits>
 
 #include "cc1d_device.hpp"
@@ -27,6 +34,7 @@ namespace {
 
 constexpr int kTileSteps = 4;                     // 64-vector steps per tile
 constexpr int kTileVecs = kTileSteps * kWave;     // 256 vectors, 4 KiB
+constexpr int kTailVecs = kWave / 4;              // most vectors 64 positions can span (fp32)
 constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
 
 typedef void __attribute__((address_space(3))) *lds_ptr_t;
@@ -34,7 +42,9 @@ typedef void __attribute__((address_space(3))) *lds_ptr_t;
 struct FwdCfTileArgs {
     uint32_t total;               // rows * tiles_per_row wavefronts
     uint32_t tiles_per_row;
-    int32_t n_vecs;               // vectors per row
+    int32_t seqlen;
+    int32_t body_vecs;            // vectors of a row that are walked as vectors (all of them, or a whole number of steps)
+    int32_t tail_vecs;            // vectors behind them, done one position per lane (0: none)
     int32_t batch, dim;
     int32_t batch_inner;          // rows numbered with the batch entry fastest
     int32_t w_dtype;
@@ -57,9 +67,10 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
     using E = Elem<DT>;
     using T = typename E::type;
     constexpr int VEC = E::kVec;
+    constexpr int EB = E::kBytes;
     constexpr bool PRECISE = E::kPreciseAct;
     constexpr bool SCALED = SILU && !PRECISE;         // taps and bias carry the factor of the SiLU exponent
-    __shared__ u32x4 lds[kBlock / kWave][kTileVecs + 1];   // [wavefront][halo vector + tile]
+    __shared__ u32x4 lds[kBlock / kWave][kTileVecs + 1 + kTailVecs];   // [wavefront][halo vector + tile + tail]
 
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     const int lane = (int)(threadIdx.x & (kWave - 1));
@@ -76,12 +87,21 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
 
     const T *xrow = reinterpret_cast<const T *>(a.x) + (int64_t)b * a.x_stride_b + (int64_t)c * a.x_stride_c;
     T *orow = reinterpret_cast<T *>(a.out) + (int64_t)b * a.out_stride_b + (int64_t)c * a.out_stride_c;
-    const int row_bytes = a.n_vecs * 16;
+    const int L = a.seqlen;
+    // The range check works on whole dwords: a 16-bit row of odd length ends in half a dword,
+    // which stays outside the resources; its element is moved separately below.
+    const int row_bytes = (L * EB) & ~3;
+    const bool odd_tail = ((L * EB) & 2) != 0;
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xrow), 0, row_bytes, kRsrcRaw);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(orow, 0, row_bytes, kRsrcRaw);
     const int v0 = tile * kTileVecs;                  // the tile's first vector
-    int steps = (a.n_vecs - v0 + kWave - 1) / kWave;  // steps of the tile that reach into the row
+    int steps = (a.body_vecs - v0 + kWave - 1) / kWave;   // steps of the tile that reach into the row
     steps = steps > kTileSteps ? kTileSteps : steps;
+    const bool last_tile = tile == (int)a.tiles_per_row - 1;
+    // A row whose last step would hold at most 64 positions ends in a tail instead: its last tile
+    // fetches those vectors too and produces their positions one per lane (an eighth of a step's
+    // instructions instead of a whole step for a handful of lanes).
+    const int tail_vecs = last_tile ? a.tail_vecs : 0;
     // LDS vector i of the wavefront holds row vector v0 - 1 + i.  For the row's first tile the
     // offset below wraps around: out of range, LDS gets zeros (the row's zero padding).
     const int vx = (lane + v0 - 1) * 16;
@@ -90,7 +110,7 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
     if (steps > 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 1024, 2);
     if (steps > 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 2048, 2);
     if (steps > 3) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 3072, 2);
-    if (lane == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(mine + steps * kWave), 16, vx + steps * 1024, 0, 0, 2);
+    if (lane < 1 + tail_vecs) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(mine + steps * kWave), 16, vx + steps * 1024, 0, 0, 2);
 
     float wv_[W], bias_v;
 #pragma unroll
@@ -113,9 +133,16 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
             init[i] = ld_elem<DT>(a.initial_states, (int64_t)b * a.init_stride_b + (int64_t)c * a.init_stride_c +
                                                         (int64_t)i * a.init_stride_l);
     }
+    // The odd last element of a 16-bit row, by the first lane of the tile that holds it.
+    const int tile_first = v0 * VEC;                  // the tile's positions start here
+    const bool holds_last = odd_tail && last_tile;
+    T last_x = T(0.f);
+    if (holds_last && lane == 0) last_x = ld_raw<DT>(xrow, L - 1);
     // Every vector of the tile is in LDS behind this wait (a vector fetched into LDS counts as a
     // load until it has been written there).
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (holds_last && lane == 0) reinterpret_cast<T *>(mine)[L - 1 + VEC - tile_first] = last_x;
+    asm volatile("" ::: "memory");                    // the element written above is read below as part of a vector
 
     for (int s = 0; s < steps; ++s) {
         float xp[VEC], xc[VEC];
@@ -139,8 +166,26 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
             for (int w = 0; w < W; ++w) s_ = fmaf(wv_[w], xx[e + w], s_);
             acc[e] = SCALED ? silu_from_scaled(s_) : SILU ? silu<PRECISE>(s_) : s_;
         }
-        // vectors behind the row's end are out of range: not stored
-        __builtin_amdgcn_raw_buffer_store_b128(E::pack(acc), ro, (lane + v0) * 16 + s * 1024, 0, 2);
+        // dwords behind the row's end are out of range: not stored
+        const u32x4 packed = E::pack(acc);
+        __builtin_amdgcn_raw_buffer_store_b128(packed, ro, (lane + v0) * 16 + s * 1024, 0, 2);
+        const int p0 = (v0 + s * kWave + lane) * VEC;  // first position of the lane's vector
+        if (odd_tail && L - 1 >= p0 && L - 1 < p0 + VEC) {
+            T o[VEC];
+            __builtin_memcpy(o, &packed, sizeof(packed));
+            st_raw<DT>(orow, L - 1, o[(L - 1) - p0]);
+        }
+    }
+
+    if (tail_vecs > 0) {
+        const int p = (v0 + steps * kWave) * VEC + lane;   // one position per lane
+        if (p < L) {
+            const T *win = reinterpret_cast<const T *>(mine) + (p + VEC - tile_first) - (W - 1);
+            float s_ = bias_v;
+#pragma unroll
+            for (int w = 0; w < W; ++w) s_ = fmaf(wv_[w], E::to_float(win[w]), s_);
+            st_elem<DT>(orow, p, SCALED ? silu_from_scaled(s_) : SILU ? silu<PRECISE>(s_) : s_);
+        }
     }
 
     // final_states[b, c, i] = x[L-(W-1)+i], copied by the wavefront of the row's FIRST tile, the
@@ -148,7 +193,6 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
     // reads are complete (the wait above) before the stores.  Rows here hold more than 64
     // vectors, so the values all come from x.
     if ((a.states & 2) != 0 && tile == 0 && lane < W - 1) {
-        const int L = a.n_vecs * VEC;
         const T v = ld_raw<DT>(xrow, L - (W - 1) + lane);
         st_raw<DT>(a.final_states, (int64_t)b * a.final_stride_b + (int64_t)c * a.final_stride_c +
                                        (int64_t)lane * a.final_stride_l, v);
@@ -174,27 +218,41 @@ int launch_tile_width(const cc1d_fwd_params &p, const FwdCfTileArgs &a, hipStrea
 
 }  // namespace
 
-// Rows of whole vectors, every row of x and of out starting on the 16-byte grid, more vectors
-// per row than the short-row kernel takes (64) and at most twice as many: there a walking
-// wavefront has one or two steps and nothing to overlap its own latency with, and tiles measured
-// 8-15 % faster ((4, 5376, 520) bf16 15.2 -> 13.1 us, (4, 5376, 768) 15.9 -> 13.8, (16, 5376, 1024)
-// 60.7 -> 55.8, (64, 2048, 1024) fp16 with states 105.7 -> 89.5 us).  Longer rows keep the walking
-// kernel, whose 256-vector segments are short-lived wavefronts already and which holds its rows in
-// registers: tiles measured 2-6 % slower there ((4, 2048, 4096) bf16 23.3 -> 23.6 us, (8, 5376, 2048)
-// 57.1 -> 59.9 us) and 16 % slower on rows that do not end on cache lines ((8, 5376, 2000) 56.5 -> 65.5 us).
+// Which launches take tiles (rows of at most 64 vectors share wavefronts in the short-row kernel).
+// Rows of whole vectors with every row of x and of out on the 16-byte grid: up to twice 64 vectors.
+// There a walking wavefront has one or two steps and nothing to overlap its own latency with, and
+// tiles measured 8-15 % faster ((4, 5376, 520) bf16 15.2 -> 13.1 us, (4, 5376, 768) 15.9 -> 13.8,
+// (16, 5376, 1024) 60.7 -> 55.8, (64, 2048, 1024) fp16 with states 105.7 -> 89.5 us).  Longer rows keep
+// the walking kernel, whose 256-vector segments are short-lived wavefronts already and which holds
+// its rows in registers: tiles measured 2-6 % slower there ((4, 2048, 4096) bf16 23.3 -> 23.6 us,
+// (8, 5376, 2048) 57.1 -> 59.9 us) and 16 % slower on rows that do not end on cache lines
+// ((8, 5376, 2000) 56.5 -> 65.5 us).
+// Rows off the grid (a length that is no whole number of vectors, a view that starts inside a
+// vector, out on another grid than x): the walking kernels do the positions outside whole vectors
+// one per lane in front of every row's walk, which costs a row of one or two steps more than the
+// row itself; a tile fetches such a row like any other.
 bool fwd_channelfirst_tile_applies(const cc1d_fwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
-    return p.seqlen % vec == 0 && p.seqlen / vec > kWave && p.seqlen / vec <= 2 * kWave &&
-           (int64_t)p.seqlen * elem_bytes(p.x_dtype) < ((int64_t)1 << 31) &&
-           aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
-           aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
+    const int64_t n_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
+    if (n_vecs <= kWave || (int64_t)p.seqlen * elem_bytes(p.x_dtype) >= ((int64_t)1 << 31) - 64) return false;
+    const bool on_grid = p.seqlen % vec == 0 &&
+                         aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
+                         aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
+    // Off the grid, tiles against the walk over rotating buffers, 16-bit: (16, 4096, 1001) bf16 49.1
+    // against 79.7 us, 1501: 69.9 / 88.9, (4, 4096, 3001): 35.9 / 42.8, 4095: 48.2 / 54.5, 8191: 101.7 / 92.5;
+    // fp32 (8, 4096, 513): 28.3 / 31.2, 1001: 54.3 / 52.4, 2047: 108.2 / 94.7.
+    return n_vecs <= (on_grid ? 2 * kWave : p.x_dtype == CC1D_F32 ? 3 * kWave : 8 * kWave);
 }
 
 int launch_fwd_channelfirst_tile(const cc1d_fwd_params &p, hipStream_t stream) {
     const int vec = vec_elems(p.x_dtype);
     FwdCfTileArgs a = {};
-    a.n_vecs = p.seqlen / vec;
-    a.tiles_per_row = (uint32_t)((a.n_vecs + kTileVecs - 1) / kTileVecs);
+    a.seqlen = p.seqlen;
+    const int n_vecs = (int)(((int64_t)p.seqlen + vec - 1) / vec);
+    const int rem = n_vecs % kWave;
+    a.tail_vecs = rem > 0 && rem * vec <= kWave ? rem : 0;
+    a.body_vecs = n_vecs - a.tail_vecs;
+    a.tiles_per_row = (uint32_t)((a.body_vecs + kTileVecs - 1) / kTileVecs);
     const int64_t total = (int64_t)p.batch * p.dim * a.tiles_per_row;
     if (total >= wave_limit()) return CC1D_ERR_TOO_LARGE;
     a.total = (uint32_t)total;

@@ -1,6 +1,7 @@
 """The channel-first tile kernels (rows fetched straight into LDS through per-row buffer
 resources): backward for every row longer than 64 vectors, at any length and alignment; forward
-for rows of 65 to 128 whole vectors on the 16-byte grid.
+for rows of 65 to 128 whole vectors on the 16-byte grid and for longer rows off that grid (a length
+that is no whole number of vectors, a view that starts inside a vector, out on another grid).
 
 Checked against the CPU oracle (tolerances of test_fwd_gpu.py / test_bwd_gpu.py) and, bit for
 bit, against the walking kernels, which a launch tunable brings back for the same tensors
@@ -8,8 +9,9 @@ bit, against the walking kernels, which a launch tunable brings back for the sam
 on which kernel produced them; dweight / dbias are sums in another order and get the oracle's
 tolerance.  Lengths: one and two elements off the vector grid on either side (1001, 1023, 1025,
 2047 -- rows that used to cost the backward twice the time of their neighbours), rows that end
-inside a tile's first and last step, one tile and several, and views that start one element
-into an allocation.
+inside a tile's first and last step, rows that end in a tail of one position per lane (516, 1025,
+1032, 2049, 2113, 4099, 4161: at most 64 positions behind a whole number of steps), one tile and
+several, and views that start one element into an allocation.
 """
 import ctypes
 
@@ -56,7 +58,7 @@ def _bwd(lib, dev, x, w, b, dout, init, dfin, shift, walking):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d)[6:])
-@pytest.mark.parametrize("seqlen", [516, 1000, 1001, 1023, 1025, 2047, 2050, 2561, 4099])
+@pytest.mark.parametrize("seqlen", [516, 1000, 1001, 1023, 1025, 1032, 2047, 2049, 2050, 2113, 2561, 4099, 4161])
 def test_bwd_rows_of_any_length_and_alignment(gpu_device, cc1d_lib, seqlen, dtype):
     lib = cabi.declare(cc1d_lib)
     g = gen(7000 + seqlen)
@@ -155,3 +157,49 @@ def test_fwd_tile_rows(pkg, gpu_device, cc1d_lib, vecs, dtype):
     assert_close(outs[0][0], ref, dtype, "out")
     assert torch.equal(outs[0][1], ref_fin)
     assert_close(outs[0][2], ref_plain, dtype, "out without activation")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d)[6:])
+@pytest.mark.parametrize("seqlen", [513, 517, 1001, 1023, 1025, 1032, 1087, 2047, 2049, 2113, 3001])
+def test_fwd_rows_off_the_grid(pkg, gpu_device, cc1d_lib, seqlen, dtype):
+    """Rows that are no whole number of vectors, or start inside one: tile kernel against the
+    walking kernels (bit for bit) and the oracle.  Lengths one and two elements off the grid on
+    either side, rows that end in a tail of one position per lane (1025, 1032, 2049, 2113), rows
+    of one tile and two, views one and three elements into their allocation, out on another
+    grid than x."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    if dtype == torch.float32 and seqlen > 3 * 64 * vec:
+        pytest.skip("fp32 rows this long keep the walking kernel")
+    g = gen(9000 + seqlen)
+    B, D, W = 3, 20, 2 + seqlen % 3
+    x = torch.randn(B, D, seqlen, generator=g).to(dtype)
+    w, b = make_wb(D, W, True, g)
+    init = make_states(B, D, W - 1, dtype, g)
+    ref, ref_fin = orc.fwd(x, w, b, initial_states=init, return_final_states=True, activation="silu")
+    ref_plain = orc.fwd(x, w, b, activation=None)
+    wd, bd, idev = w.to(dev), b.to(dev), init.to(dev)
+    for x_shift, out_shift in ((0, 0), (1, 1), (3, 0), (0, 2)):
+        xd = _view(x, dev, x_shift)
+        got = []
+        try:
+            for knob in (0, -1):
+                assert lib.cc1d_set_tunable(b"fwd_cf_vecs", knob) == 0
+                out = _view(torch.zeros_like(x), dev, out_shift)
+                fin = torch.empty(B, W - 1, D, dtype=dtype, device=dev).transpose(1, 2)
+                p = cabi.fwd_params(xd, wd, bd, out, True, initial_states=idev, final_states=fin)
+                assert lib.cc1d_fwd(ctypes.byref(p), None) == 0
+                out2 = _view(torch.zeros_like(x), dev, out_shift)
+                p2 = cabi.fwd_params(xd, wd, bd, out2, False)
+                assert lib.cc1d_fwd(ctypes.byref(p2), None) == 0
+                torch.cuda.synchronize()
+                got.append((out.cpu(), fin.cpu(), out2.cpu()))
+        finally:
+            lib.cc1d_set_tunable(b"fwd_cf_vecs", 0)
+        what = "seqlen %d x shift %d out shift %d" % (seqlen, x_shift, out_shift)
+        for a, r in zip(got[0], got[1]):
+            assert torch.equal(a, r), "tile and walking kernels differ, " + what
+        assert_close(got[0][0], ref, dtype, "out, " + what)
+        assert torch.equal(got[0][1], ref_fin), what
+        assert_close(got[0][2], ref_plain, dtype, "out without activation, " + what)
