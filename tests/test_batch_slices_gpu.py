@@ -16,6 +16,8 @@ from oracle import causal_conv1d_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
+TOO_LARGE = -16                     # CC1D_ERR_TOO_LARGE (include/cc1d.h)
+
 
 class _Limit:
     """Context manager: one launch holds at most 2^(31 - shift) threads."""
@@ -134,3 +136,91 @@ def test_update_in_batch_slices(pkg, gpu_device, cc1d_lib, circular, unit_stride
     for shift in (21, 22):
         got = run(shift)
         assert torch.equal(got[0], whole[0]) and torch.equal(got[1], whole[1])
+
+
+@pytest.mark.parametrize("layout", ["step", "tokens", "rowstate"])
+@pytest.mark.parametrize("circular", [False, True])
+def test_decode_step_in_batch_slices(pkg, gpu_device, cc1d_lib, layout, circular):
+    """The decode-step launchers proper: one token on a cache with unit stride along dim (step
+    kernel), four tokens (multi-token kernel), one token on a contiguous (batch, dim, state_len)
+    cache (row-state kernel).  Each answers "too large" against the lowered ceiling and the
+    front slices the batch; out and conv_state must equal the single launch bit for bit."""
+    if layout == "rowstate" and circular:
+        pytest.skip("the row-state kernel shifts its cache; ring buffers take the other kernels")
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    g = gen(91)
+    B, D, W = 37, 256, 4
+    S = 4 if layout == "rowstate" else 8 if circular else 3
+    seqlen = 4 if layout == "tokens" else 1
+    x = torch.randn(B, seqlen, D, generator=g).to(torch.bfloat16).transpose(1, 2).to(dev)
+    if layout == "rowstate":
+        state0 = torch.randn(B, D, S, generator=g).to(torch.bfloat16).to(dev)
+        x = x.contiguous()
+    else:
+        state0 = torch.randn(B, S, D, generator=g).to(torch.bfloat16).transpose(1, 2).to(dev)
+    w, b = (t.to(dev) for t in make_wb(D, W, True, g))
+    cs = torch.randint(0, 1000, (B,), generator=g, dtype=torch.int32).to(dev) if circular else None
+
+    def run(shift):
+        st = state0.clone() if layout == "rowstate" else state0.transpose(1, 2).clone().transpose(1, 2)
+        with _Limit(lib, shift):
+            out = pkg.causal_conv1d_update(x, st, w, b, activation="silu", cache_seqlens=cs)
+        return out, st
+
+    whole = run(0)
+    ref_state = state0.cpu().clone()
+    ref = orc.update(x.cpu(), ref_state, w.cpu(), b.cpu(), activation="silu",
+                     cache_seqlens=None if cs is None else cs.cpu())
+    assert_close(whole[0], ref, torch.bfloat16, "out")
+    assert torch.equal(whole[1].cpu(), ref_state)
+    # the whole batch is 1280 threads (step: 64 lanes x 4 channels a block row, 8 batch entries a
+    # block), about as many (tokens), 5120 (row-state: 128 channels x 4 batch entries a block);
+    # the ceilings leave a few blocks, or one, to a launch
+    for shift in {"step": (21, 22), "tokens": (21, 22), "rowstate": (19, 20, 21)}[layout]:
+        got = run(shift)
+        assert torch.equal(got[0], whole[0]) and torch.equal(got[1], whole[1]), "shift %d" % shift
+
+
+def test_flat_forward_in_batch_slices(pkg, gpu_device, cc1d_lib):
+    """Contiguous channel-first rows that are no whole number of vectors (the flat kernel reads the
+    tensor as one array): sliced along the batch against the single launch."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    g = gen(92)
+    B, D, L = 11, 136, 100
+    x = torch.randn(B, D, L, generator=g).to(torch.bfloat16).to(dev)
+    w, b = (t.to(dev) for t in make_wb(D, 4, True, g))
+    whole = pkg.causal_conv1d_fn(x, w, b, activation="silu")
+    for shift in (15, 17):                              # 65536 and 16384 threads to a launch; the tensor has 149600 elements
+        with _Limit(lib, shift):
+            got = pkg.causal_conv1d_fn(x, w, b, activation="silu")
+        assert torch.equal(got, whole), "shift %d" % shift
+    assert_close(whole, orc.fwd(x.cpu(), w.cpu(), b.cpu(), activation="silu"), torch.bfloat16, "out")
+
+
+def test_a_batch_entry_too_large_is_refused_before_anything_runs(gpu_device, cc1d_lib):
+    """When even one batch entry exceeds the ceiling no slicing can help: the call answers
+    CC1D_ERR_TOO_LARGE and has launched nothing -- out, dx, dweight keep what they held."""
+    lib = cabi.declare(cc1d_lib)
+    dev = gpu_device
+    g = gen(93)
+    B, D, L = 6, 136, 700
+    for channel_last in (False, True):
+        x = make_x(B, D, L, torch.bfloat16, channel_last, g, sliced=False).to(dev)
+        dout = make_x(B, D, L, torch.bfloat16, channel_last, g, sliced=False).to(dev)
+        w, b = (t.to(dev) for t in make_wb(D, 4, True, g))
+        out = torch.full_like(x, 7.0)
+        dx = torch.full_like(x, 7.0)
+        dw, db = torch.full((D, 4), 7.0, device=dev), torch.full((D,), 7.0, device=dev)
+        pf = cabi.fwd_params(x, w, b, out, True)
+        pb = cabi.bwd_params(x, w, b, dout, dx, dw, db, True)
+        with _Limit(lib, 24):                           # 128 threads to a launch: less than one batch entry needs
+            assert lib.cc1d_fwd(ctypes.byref(pf), None) == TOO_LARGE
+            need = ctypes.c_size_t()
+            st = lib.cc1d_bwd_workspace_bytes(ctypes.byref(pb), ctypes.byref(need))
+            ws = torch.empty(max(16, need.value if st == 0 else 1 << 20), dtype=torch.uint8, device=dev)
+            assert lib.cc1d_bwd(ctypes.byref(pb), ws.data_ptr(), ws.numel(), None) == TOO_LARGE
+        torch.cuda.synchronize()
+        for t in (out, dx, dw, db):
+            assert bool((t == 7.0).all()), "a refused call wrote to its outputs"
