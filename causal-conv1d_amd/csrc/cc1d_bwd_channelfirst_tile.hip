@@ -42,8 +42,7 @@
 namespace cc1d {
 namespace {
 
-constexpr int kTileSteps = 4;                     // 64-vector steps per tile
-constexpr int kTileVecs = kTileSteps * kWave;     // 256 vectors, 4 KiB per tensor
+constexpr int kTileSteps = 4;                     // most 64-vector steps a tile has (256 vectors, 4 KiB per tensor)
 constexpr int kTailVecs = kWave / 4;              // most vectors 64 positions can span (fp32)
 constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
 
@@ -52,6 +51,7 @@ typedef void __attribute__((address_space(3))) *lds_ptr_t;
 struct BwdCfTileArgs {
     uint32_t total;               // rows * tiles_per_row wavefronts
     uint32_t tiles_per_row;
+    int32_t steps_per_tile;       // 64-vector steps of every tile but a row's last, which may have fewer (1 .. 4)
     int32_t seqlen;
     int32_t body_vecs;            // vectors of a row that are walked as vectors (all of them, or a whole number of steps)
     int32_t tail_vecs;            // vectors behind them, done one position per lane (0: none)
@@ -94,8 +94,9 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     constexpr int VEC = E::kVec;
     constexpr int EB = E::kBytes;
     constexpr bool PRECISE = E::kPreciseAct;
-    constexpr int XV = kTileVecs + 2 + kTailVecs, DV = kTileVecs + 1 + kTailVecs;   // vectors of x and of dout a tile holds
-    __shared__ u32x4 lds[kBlock / kWave][XV + DV];
+    extern __shared__ u32x4 lds[];                    // [wavefront][x vectors | dout vectors]
+    const int tile_vecs = a.steps_per_tile * kWave;
+    const int XV = tile_vecs + 2 + kTailVecs, DV = tile_vecs + 1 + kTailVecs;   // vectors of x and of dout a tile holds
 
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     const int lane = (int)(threadIdx.x & (kWave - 1));
@@ -118,16 +119,16 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(xrow), 0, row_bytes, kRsrcRaw);
     const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(drow), 0, row_bytes, kRsrcRaw);
     const __amdgpu_buffer_rsrc_t rdx = __builtin_amdgcn_make_buffer_rsrc(dxrow, 0, row_bytes, kRsrcRaw);
-    const int v0 = tile * kTileVecs;                  // the tile's first vector
+    const int v0 = tile * tile_vecs;                  // the tile's first vector
     int steps = (a.body_vecs - v0 + kWave - 1) / kWave;   // steps of the tile that reach into the row
-    steps = steps > kTileSteps ? kTileSteps : steps;
+    steps = steps > a.steps_per_tile ? a.steps_per_tile : steps;
     // A row whose last step would hold at most 64 positions ends in a tail instead: its last tile
     // fetches those vectors too and takes their positions one per lane (an eighth of a step's
     // instructions instead of a whole step for a handful of lanes).
     const int tail_vecs = tile == (int)a.tiles_per_row - 1 ? a.tail_vecs : 0;
     // x vector i of the wavefront's LDS holds row vector v0 - 1 + i, dout vector i holds v0 + i.
     // For the row's first tile the x offset below wraps around: out of range, zeros.
-    u32x4 *xl = &lds[wv][0], *dl = &lds[wv][XV];
+    u32x4 *xl = lds + wv * (XV + DV), *dl = xl + XV;
     const int vx = (lane + v0 - 1) * 16, vd = (lane + v0) * 16;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 0, 2);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 0, 2);
@@ -323,8 +324,10 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
 template <int DT, int W>
 int launch_tile_act(const cc1d_bwd_params &p, const BwdCfTileArgs &a, hipStream_t stream) {
     const uint32_t blocks = (a.total + (kBlock / kWave) - 1) / (kBlock / kWave);
-    if (p.silu) CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, a);
-    else CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, a);
+    // per wavefront: steps_per_tile steps of x and of dout, the vectors around them, room for a tail
+    const size_t lds = (size_t)(kBlock / kWave) * (2 * a.steps_per_tile * kWave + 3 + 2 * kTailVecs) * sizeof(u32x4);
+    if (p.silu) CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), lds, stream, a);
+    else CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), lds, stream, a);
     return launch_status();
 }
 
@@ -344,10 +347,19 @@ int tail_vecs_of_row(const cc1d_bwd_params &p) {
     return rem > 0 && rem * vec <= kWave ? rem : 0;
 }
 
-int64_t tiles_per_row(const cc1d_bwd_params &p) {
+// A row's steps are dealt to as few tiles of at most four steps as hold them, evenly (five steps:
+// 3 + 2, not 4 + 1): a tile's LDS is sized for steps_per_tile, and the fewer it holds the more
+// wavefronts fit a CU -- (16, 4096, 1024) bf16, two steps a row: 80.4 -> 75.7 us with LDS for two
+// steps instead of four.
+int64_t steps_of_row(const cc1d_bwd_params &p) {
     const int vec = vec_elems(p.x_dtype);
     const int64_t body_vecs = ((int64_t)p.seqlen + vec - 1) / vec - tail_vecs_of_row(p);
-    return (body_vecs + kTileVecs - 1) / kTileVecs;
+    return (body_vecs + kWave - 1) / kWave;
+}
+int64_t tiles_per_row(const cc1d_bwd_params &p) { return (steps_of_row(p) + kTileSteps - 1) / kTileSteps; }
+int steps_per_tile(const cc1d_bwd_params &p) {
+    const int64_t tiles = tiles_per_row(p);
+    return (int)((steps_of_row(p) + tiles - 1) / tiles);
 }
 
 }  // namespace
@@ -369,6 +381,7 @@ int launch_bwd_channelfirst_tile(const cc1d_bwd_params &p, float *ws, hipStream_
     if (!bwd_channelfirst_tile_fits(p)) return CC1D_ERR_TOO_LARGE;
     BwdCfTileArgs a = {};
     a.tiles_per_row = (uint32_t)tiles_per_row(p);
+    a.steps_per_tile = steps_per_tile(p);
     a.total = (uint32_t)((int64_t)p.batch * p.dim * a.tiles_per_row);
     a.seqlen = p.seqlen; a.batch = p.batch; a.dim = p.dim;
     a.tail_vecs = tail_vecs_of_row(p);
