@@ -366,9 +366,13 @@ int launch_taps(const FwdClArgs &a, const FwdClRare &q, int width, bool silu, in
 // holds, and hold less LDS, so more of them are in flight.  Measured at the prefill shape
 // (8, 5376, 2048) bf16, the same buffers every launch / six rotating sets: 8 rows 64.7 / 62.7 us,
 // 16 rows 56.1 / 55.9, 24 rows 57.8 / 57.5, 32 rows 58.5 / 58.3.
-static int choose_rows_per_run(int seqlen, int64_t row_bytes, int width) {
+// Launches of at most 1536 wavefronts (a fifth of what the chip holds: a prompt of a few dozen
+// tokens, a short chunk of a prefill) are bound by one wavefront's chain of fetch, walk and store
+// and take runs of 8 rows: (1, 5376, 64) bf16 4.65 -> 4.05 us, (4, 5376, 128) 5.19 -> 4.70,
+// (1, 5376, 512) 5.16 -> 4.65; at 2048 wavefronts and more 16 rows are as fast or faster.
+static int choose_rows_per_run(int seqlen, int64_t row_bytes, int width, int64_t waves_at_default) {
     int T = tunables().fwd_cl_rows;
-    if (T <= 0) T = kDefaultRows;
+    if (T <= 0) T = waves_at_default <= 1536 ? kGroup : kDefaultRows;
     const int cap = (seqlen + kGroup - 1) / kGroup * kGroup;      // never longer than the sequence
     if (T > cap) T = cap;
     T = (T + kGroup - 1) / kGroup * kGroup;
@@ -390,7 +394,8 @@ int launch_fwd_channellast(const cc1d_fwd_params &p, const cc1d_varlen_params *g
     a.n_cols = p.dim / ch;
     const int64_t row_stride = p.x_stride_l > p.out_stride_l ? p.x_stride_l : p.out_stride_l;
     a.waves_per_row = (uint32_t)((a.n_cols + kWave - 1) / kWave);
-    a.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * eb, p.width);
+    a.rows_per_run = choose_rows_per_run(p.seqlen, row_stride * eb, p.width,
+                                         (int64_t)p.batch * ((p.seqlen + kDefaultRows - 1) / kDefaultRows) * a.waves_per_row);
     if (a.rows_per_run == 0) return CC1D_ERR_TOO_LARGE;
     a.n_runs = (p.seqlen + a.rows_per_run - 1) / a.rows_per_run;
     const int64_t total = (int64_t)p.batch * a.n_runs * a.waves_per_row;
