@@ -9,10 +9,12 @@
 //   dweight[w] += sum_{b,t} g[t] * xpad[t-(W-1-w)],   dbias += sum_{b,t} g[t]
 //
 // Design.  A wavefront takes a tile of up to four 64-vector steps of one (batch, channel) row
-// and asks for all of its x and dout at once; the data goes from memory straight into LDS
-// (buffer_load_dwordx4 ... lds) together with the vector in front of the tile (the x halo) and
-// the vectors behind it (x and dout of the W-1 positions whose g the tile's last lane needs).
-// No registers are held while the tile is in flight, so the launch is thousands of wavefronts
+// and asks for all of its x and dout at once.  x goes from memory straight into LDS
+// (buffer_load_dwordx4 ... lds), where a lane finds its neighbours' elements, together with the
+// vector in front of the tile (the x halo) and the vectors behind it (the W-1 positions whose g
+// the tile's last lane needs); dout, which only the lane that owns it reads, goes to registers
+// (four per step: with LDS for one tensor instead of two, seven wavefronts share a SIMD instead
+// of four: 1-3 % at most shapes, (2, 2048, 16384) bf16 71.1 -> 69.2 us).  The launch is thousands of wavefronts
 // that live for one memory round trip and a few hundred instructions each and sweep through
 // memory as one compact front in the order of the rows -- where one long-lived wavefront per
 // channel walks 4096 far-apart streams at once, which is what bounds that design at the
@@ -42,7 +44,10 @@
 namespace cc1d {
 namespace {
 
-constexpr int kTileSteps = 4;                     // most 64-vector steps a tile has (256 vectors, 4 KiB per tensor)
+// Most 64-vector steps a tile has (256 vectors, 4 KiB per tensor).  Fewer cost more wavefronts, each
+// with its taps, its g values behind the tile and its reduction (fp16 (4, 4096, 8192): three steps
+// 145 us, two 150 us against 140 us); six and eight measured no better than four.
+constexpr int kTileSteps = 4;
 constexpr int kTailVecs = kWave / 4;              // most vectors 64 positions can span (fp32)
 constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
 
@@ -94,9 +99,9 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     constexpr int VEC = E::kVec;
     constexpr int EB = E::kBytes;
     constexpr bool PRECISE = E::kPreciseAct;
-    extern __shared__ u32x4 lds[];                    // [wavefront][x vectors | dout vectors]
+    extern __shared__ u32x4 lds[];                    // [wavefront][x vectors]
     const int tile_vecs = a.steps_per_tile * kWave;
-    const int XV = tile_vecs + 2 + kTailVecs, DV = tile_vecs + 1 + kTailVecs;   // vectors of x and of dout a tile holds
+    const int XV = tile_vecs + 2 + kTailVecs;         // vectors of x a tile holds
 
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     const int lane = (int)(threadIdx.x & (kWave - 1));
@@ -126,28 +131,41 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     // fetches those vectors too and takes their positions one per lane (an eighth of a step's
     // instructions instead of a whole step for a handful of lanes).
     const int tail_vecs = tile == (int)a.tiles_per_row - 1 ? a.tail_vecs : 0;
-    // x vector i of the wavefront's LDS holds row vector v0 - 1 + i, dout vector i holds v0 + i.
-    // For the row's first tile the x offset below wraps around: out of range, zeros.
-    u32x4 *xl = lds + wv * (XV + DV), *dl = xl + XV;
+    // x goes to LDS, where a lane finds its neighbours' elements: vector i of the wavefront's LDS
+    // holds row vector v0 - 1 + i (for the row's first tile the offset below wraps around: out of
+    // range, zeros).  dout is needed by the lane that owns it only and goes to registers: LDS for
+    // one tensor instead of two lets twice as many wavefronts share a CU.
+    u32x4 *xl = lds + wv * XV;
     const int vx = (lane + v0 - 1) * 16, vd = (lane + v0) * 16;
+    u32x4 dreg[kTileSteps];
+#pragma unroll
+    for (int s = 0; s < kTileSteps; ++s) dreg[s] = u32x4{0u, 0u, 0u, 0u};
+    // Step s: the lane's offset in the vector register, s KiB as the instruction's immediate
+    // offset, which the hardware adds to the LDS address as well, so the LDS pointer stays put.
+    // (A scalar offset would do for the address but is left out of the range check, which the
+    // row's ends rely on.)
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 0, 2);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 0, 2);
+    dreg[0] = __builtin_amdgcn_raw_buffer_load_b128(rd, vd, 0, 2);
     if (steps > 1) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 1024, 2);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 1024, 2);
+        dreg[1] = __builtin_amdgcn_raw_buffer_load_b128(rd, vd + 1024, 0, 2);
     }
     if (steps > 2) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 2048, 2);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 2048, 2);
+        dreg[2] = __builtin_amdgcn_raw_buffer_load_b128(rd, vd + 2048, 0, 2);
     }
     if (steps > 3) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)xl, 16, vx, 0, 3072, 2);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)dl, 16, vd, 0, 3072, 2);
+        dreg[3] = __builtin_amdgcn_raw_buffer_load_b128(rd, vd + 3072, 0, 2);
     }
-    // behind the tile: two more vectors of x, one of dout (what the top step's last lane needs),
-    // and the row's tail
+    // behind the tile: two more vectors of x and the row's tail; the one vector of dout behind the
+    // tile (what the top step's last lane needs) is the same for every lane
     if (lane < 2 + tail_vecs) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(xl + steps * kWave), 16, vx + steps * 1024, 0, 0, 0);
-    if (lane < 1 + tail_vecs) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (lds_ptr_t)(dl + steps * kWave), 16, vd + steps * 1024, 0, 0, 0);
+    const u32x4 dbehind = __builtin_amdgcn_raw_buffer_load_b128(rd, (v0 + steps * kWave) * 16, 0, 0);
+    // the tail's dout, one position per lane
+    const int p_tail = (v0 + steps * kWave) * VEC + lane;
+    T tail_d = T(0.f);
+    if (tail_vecs > 0 && p_tail < L) tail_d = ld_raw<DT>(drow, p_tail);
 
     // Taps and bias of the channel (wave-uniform); with the fast activation also times -log2(e),
     // so that the sum over the window is the exponent the derivative needs.
@@ -165,9 +183,9 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     const int tile_first = v0 * VEC, tile_end = (v0 + steps * kWave + tail_vecs) * VEC;   // positions [tile_first, tile_end)
     const bool holds_last = odd_tail && L - 1 >= tile_first - VEC && L - 1 < tile_end + VEC;
     T last_x = T(0.f), last_d = T(0.f);
-    if (holds_last && lane == 0) {
-        last_x = ld_raw<DT>(xrow, L - 1);
-        last_d = ld_raw<DT>(drow, L - 1);
+    if (holds_last) {
+        if (lane == 0) last_x = ld_raw<DT>(xrow, L - 1);
+        last_d = ld_raw<DT>(drow, L - 1);             // every lane: the lane that owns the position patches its vector
     }
     T init_raw[W - 1];
     const bool has_init = a.initial_states != nullptr && tile == 0;
@@ -193,10 +211,9 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
     // load until it has been written there).
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (holds_last && lane == 0) {
-        // LDS element index of row position p: x region (p + VEC - tile_first), dout region (p - tile_first)
-        const int ix = L - 1 + VEC - tile_first, id = L - 1 - tile_first;
+        // LDS element index of row position p: p + VEC - tile_first
+        const int ix = L - 1 + VEC - tile_first;
         if (ix >= 0 && ix < XV * VEC) reinterpret_cast<T *>(xl)[ix] = last_x;
-        if (id >= 0 && id < DV * VEC) reinterpret_cast<T *>(dl)[id] = last_d;
     }
     if (has_init && lane == 0) {
 #pragma unroll
@@ -219,7 +236,7 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
         float xw[W];
 #pragma unroll
         for (int k = 0; k < W; ++k) xw[k] = in_row ? E::to_float(xe[k]) : 0.f;
-        const float dv = in_row ? E::to_float(reinterpret_cast<const T *>(dl)[p - tile_first]) : 0.f;
+        const float dv = in_row ? E::to_float(tail_d) : 0.f;
         float g[W];
         g[0] = SILU ? __builtin_fmaf(dv, act_grad(xw), 0.f) : dv;
 #pragma unroll
@@ -242,7 +259,7 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
         float xa[VEC], xb[VEC], dv[VEC];
         E::unpack(xl[steps * kWave], xa);
         E::unpack(xl[steps * kWave + 1], xb);
-        E::unpack(dl[steps * kWave], dv);
+        E::unpack(dbehind, dv);
         float xwin[2 * (W - 1)];
 #pragma unroll
         for (int i = 0; i < W - 1; ++i) { xwin[i] = xa[VEC - (W - 1) + i]; xwin[W - 1 + i] = xb[i]; }
@@ -250,11 +267,19 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
         for (int e = 0; e < W - 1; ++e) carry[e] = SILU ? __builtin_fmaf(dv[e], act_grad(&xwin[e]), 0.f) : dv[e];
     }
 
-    for (int s = steps - 1; s >= 0; --s) {
+#pragma unroll
+    for (int s = kTileSteps - 1; s >= 0; --s) {
+        if (s >= steps) continue;
         float xp[VEC], xc[VEC], dv[VEC];
         E::unpack(xl[s * kWave + lane], xp);
         E::unpack(xl[s * kWave + lane + 1], xc);
-        E::unpack(dl[s * kWave + lane], dv);
+        E::unpack(dreg[s], dv);
+        const int p0 = (v0 + s * kWave + lane) * VEC;      // first position of the lane's vector
+        const int step_first = (v0 + s * kWave) * VEC;
+        if (holds_last && L - 1 >= step_first && L - 1 < step_first + kWave * VEC) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) dv[e] = p0 + e == L - 1 ? E::to_float(last_d) : dv[e];
+        }
         // xw[i] = padded x at position (first position of the lane's vector) - (W-1) + i
         float xw[VEC + W - 1], g[VEC + W - 1];
 #pragma unroll
@@ -278,8 +303,6 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
 #pragma unroll
             for (int k = 0; k < W; ++k) dW[k] = fmaf(g[e], xw[e + k], dW[k]);
         }
-        const int p0 = (v0 + s * kWave + lane) * VEC;      // first position of the lane's vector
-        const int step_first = (v0 + s * kWave) * VEC;
         if (has_dfinal && L - 1 >= step_first && L - (W - 1) < step_first + kWave * VEC) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
@@ -324,8 +347,8 @@ bwd_channelfirst_tile_kernel(const BwdCfTileArgs a) {
 template <int DT, int W>
 int launch_tile_act(const cc1d_bwd_params &p, const BwdCfTileArgs &a, hipStream_t stream) {
     const uint32_t blocks = (a.total + (kBlock / kWave) - 1) / (kBlock / kWave);
-    // per wavefront: steps_per_tile steps of x and of dout, the vectors around them, room for a tail
-    const size_t lds = (size_t)(kBlock / kWave) * (2 * a.steps_per_tile * kWave + 3 + 2 * kTailVecs) * sizeof(u32x4);
+    // per wavefront: steps_per_tile steps of x, the vectors around them, room for a tail
+    const size_t lds = (size_t)(kBlock / kWave) * (a.steps_per_tile * kWave + 2 + kTailVecs) * sizeof(u32x4);
     if (p.silu) CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), lds, stream, a);
     else CC1D_LAUNCH((bwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), lds, stream, a);
     return launch_status();
