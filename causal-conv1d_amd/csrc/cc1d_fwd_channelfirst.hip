@@ -27,10 +27,10 @@
 // produced one per lane, straight from memory.  The general kernel takes out tensors on a different grid.  The short-row
 // kernel takes rows of at most 64 vectors, several rows to a wavefront and no walk; the flat
 // kernel takes such rows of a contiguous tensor as whole vectors of one flat array.  Rows of
-// 65 to 128 whole vectors on the 16-byte grid, and rows off that grid of up to 512 vectors (192
-// of fp32), go to the tile kernel of cc1d_fwd_channelfirst_tile.hip (rows fetched straight into
-// LDS; 8-15 % faster on the grid, 10-40 % off it, slower than the walk for longer rows); the
-// launch tunable fwd_cf_vecs = -1 keeps them here.
+// more than 64 vectors that start on 128-byte lines (tensors of up to 512 MiB) or hold at most
+// 128 vectors, and rows off the 16-byte grid of up to 512 vectors (192 of fp32), go to the tile
+// kernel of cc1d_fwd_channelfirst_tile.hip (rows fetched straight into LDS; 1-25 % faster on
+// lines, 10-40 % off the grid); the launch tunable fwd_cf_vecs = -1 keeps them here.
 #include <type_traits>
 
 #include "cc1d_device.hpp"

@@ -1,7 +1,7 @@
 // Channel-first forward for gfx950: short-lived tile wavefronts.  Takes over
-// causal_conv1d_fwd_kernel (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for rows of 65 to
-// 128 whole 16-byte vectors on the 16-byte grid (a contiguous (batch, dim, seqlen) tensor with
-// seqlen 520 .. 1024 in 16-bit data, 260 .. 512 in fp32) and for rows off that grid -- a length
+// causal_conv1d_fwd_kernel (csrc/causal_conv1d_fwd.cu:46-170 of the reference) for rows of more
+// than 64 sixteen-byte vectors: rows of whole vectors on the 16-byte grid that start on 128-byte
+// lines (tensors of up to 512 MiB) or hold at most 128 vectors, and rows off that grid -- a length
 // that is no whole number of vectors, a view that starts inside a vector, out on another grid
 // than x -- of up to 512 vectors of 16-bit data, 192 of fp32.  Everything else stays with the
 // kernels of cc1d_fwd_channelfirst.hip (see fwd_channelfirst_tile_applies below for the
@@ -219,29 +219,36 @@ int launch_tile_width(const cc1d_fwd_params &p, const FwdCfTileArgs &a, hipStrea
 }  // namespace
 
 // Which launches take tiles (rows of at most 64 vectors share wavefronts in the short-row kernel).
-// Rows of whole vectors with every row of x and of out on the 16-byte grid: up to twice 64 vectors.
-// There a walking wavefront has one or two steps and nothing to overlap its own latency with, and
-// tiles measured 8-15 % faster ((4, 5376, 520) bf16 15.2 -> 13.1 us, (4, 5376, 768) 15.9 -> 13.8,
-// (16, 5376, 1024) 60.7 -> 55.8, (64, 2048, 1024) fp16 with states 105.7 -> 89.5 us).  Longer rows keep
-// the walking kernel, whose 256-vector segments are short-lived wavefronts already and which holds
-// its rows in registers: tiles measured 2-6 % slower there ((4, 2048, 4096) bf16 23.3 -> 23.6 us,
-// (8, 5376, 2048) 57.1 -> 59.9 us) and 16 % slower on rows that do not end on cache lines
-// ((8, 5376, 2000) 56.5 -> 65.5 us).
-// Rows off the grid (a length that is no whole number of vectors, a view that starts inside a
-// vector, out on another grid than x): the walking kernels do the positions outside whole vectors
-// one per lane in front of every row's walk, which costs a row of one or two steps more than the
-// row itself; a tile fetches such a row like any other.
+// Over rotating buffer sets, tiles against the walking kernel, us:
+//  * rows of whole vectors on the 16-byte grid, up to twice 64 vectors: a walking wavefront has one
+//    or two steps and nothing to overlap its own latency with; (4, 5376, 520) bf16 13.1 / 15.2,
+//    (16, 5376, 1024) 55.8 / 60.7, (64, 2048, 1024) fp16 with states 89.5 / 105.7;
+//  * longer rows when every row of x and of out starts on a 128-byte line and a tensor holds at
+//    most 512 MiB: (4, 2048, 4096) bf16 24.2 / 25.1, fp32 43.2 / 44.1, (8, 5376, 2048) bf16 56.8 / 58.2,
+//    (1, 5376, 2048) 10.0 / 11.2, (2, 1024, 2048) 5.3 / 7.0.  Beyond that size the walk, whose
+//    wavefronts are fewer and longer-lived, is ahead ((64, 5376, 2048) bf16 459.8 / 448.0), and so it is
+//    for rows on the grid that do not start on lines, where it moves the steps of a row onto the
+//    lines of out and a tile cannot ((8, 5376, 3000) bf16 90.6 / 83.7, (8, 5376, 1500) fp32 88.6 / 83.6);
+//  * rows off the grid (a length that is no whole number of vectors, a view that starts inside a
+//    vector, out on another grid than x), up to 512 vectors of 16-bit data and 192 of fp32: the
+//    walking kernels do the positions outside whole vectors one per lane in front of every row's
+//    walk, which costs a row of one or two steps more than the row itself; (16, 4096, 1001) bf16
+//    49.1 / 79.7, 1501: 69.9 / 88.9, (4, 4096, 4095) 48.2 / 54.5, 8191: 101.7 / 92.5; fp32 (8, 4096, 513)
+//    28.3 / 31.2, 1001: 54.3 / 52.4, 2047: 108.2 / 94.7.
 bool fwd_channelfirst_tile_applies(const cc1d_fwd_params &p) {
-    const int vec = vec_elems(p.x_dtype);
+    const int vec = vec_elems(p.x_dtype), eb = elem_bytes(p.x_dtype);
     const int64_t n_vecs = ((int64_t)p.seqlen + vec - 1) / vec;
-    if (n_vecs <= kWave || (int64_t)p.seqlen * elem_bytes(p.x_dtype) >= ((int64_t)1 << 31) - 64) return false;
+    if (n_vecs <= kWave || (int64_t)p.seqlen * eb >= ((int64_t)1 << 31) - 64) return false;
     const bool on_grid = p.seqlen % vec == 0 &&
                          aligned16(p.x) && p.x_stride_b % vec == 0 && p.x_stride_c % vec == 0 &&
                          aligned16(p.out) && p.out_stride_b % vec == 0 && p.out_stride_c % vec == 0;
-    // Off the grid, tiles against the walk over rotating buffers, 16-bit: (16, 4096, 1001) bf16 49.1
-    // against 79.7 us, 1501: 69.9 / 88.9, (4, 4096, 3001): 35.9 / 42.8, 4095: 48.2 / 54.5, 8191: 101.7 / 92.5;
-    // fp32 (8, 4096, 513): 28.3 / 31.2, 1001: 54.3 / 52.4, 2047: 108.2 / 94.7.
-    return n_vecs <= (on_grid ? 2 * kWave : p.x_dtype == CC1D_F32 ? 3 * kWave : 8 * kWave);
+    if (!on_grid) return n_vecs <= (p.x_dtype == CC1D_F32 ? 3 * kWave : 8 * kWave);
+    if (n_vecs <= 2 * kWave) return true;
+    auto on_lines = [eb](const void *base, int64_t stride_b, int64_t stride_c) {
+        return reinterpret_cast<uintptr_t>(base) % 128 == 0 && stride_b * eb % 128 == 0 && stride_c * eb % 128 == 0;
+    };
+    return on_lines(p.x, p.x_stride_b, p.x_stride_c) && on_lines(p.out, p.out_stride_b, p.out_stride_c) &&
+           (int64_t)p.batch * p.dim * p.seqlen * eb <= ((int64_t)1 << 29);
 }
 
 int launch_fwd_channelfirst_tile(const cc1d_fwd_params &p, hipStream_t stream) {

@@ -1,7 +1,8 @@
 """The channel-first tile kernels (rows fetched straight into LDS through per-row buffer
 resources): backward for every row longer than 64 vectors, at any length and alignment; forward
-for rows of 65 to 128 whole vectors on the 16-byte grid and for longer rows off that grid (a length
-that is no whole number of vectors, a view that starts inside a vector, out on another grid).
+for rows on the 16-byte grid of 65 to 128 whole vectors or starting on 128-byte lines, and for
+rows off that grid (a length that is no whole number of vectors, a view that starts inside a
+vector, out on another grid).
 
 Checked against the CPU oracle (tolerances of test_fwd_gpu.py / test_bwd_gpu.py) and, bit for
 bit, against the walking kernels, which a launch tunable brings back for the same tensors
@@ -125,10 +126,12 @@ def test_bwd_tiles_at_a_size_that_fills_the_chip(gpu_device, cc1d_lib):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d)[6:])
-@pytest.mark.parametrize("vecs", [65, 96, 127, 128])
+@pytest.mark.parametrize("vecs", [65, 96, 127, 128, 192, 256, 320, 520, 1032])
 def test_fwd_tile_rows(pkg, gpu_device, cc1d_lib, vecs, dtype):
-    """Forward rows of 65 .. 128 whole vectors: tile kernel against the walking kernel (bit for
-    bit) and the oracle, with and without states, rows as a channel slice of a wider tensor."""
+    """Forward rows of whole vectors on the 16-byte grid -- 65 .. 128 vectors, and longer rows that
+    start on 128-byte lines (one tile, two, several; 1032 vectors end in a tail) -- tile kernel
+    against the walking kernel (bit for bit) and the oracle, with and without states, rows as a
+    channel slice of a wider tensor."""
     lib = cabi.declare(cc1d_lib)
     dev = gpu_device
     vec = 16 // torch.empty(0, dtype=dtype).element_size()
