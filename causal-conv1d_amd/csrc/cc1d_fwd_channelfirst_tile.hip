@@ -11,7 +11,7 @@
 // row and asks for all of it at once: the data goes from memory straight into LDS
 // (buffer_load_dwordx4 ... lds), together with the vector in front of the tile, whose last W-1
 // elements are the tile's halo.  No registers are held while the tile is in flight, a tile needs
-// 4.1 KB of LDS, and eight wavefronts fit a SIMD; they live for one memory round trip and a few
+// 4.4 KB of LDS, and eight wavefronts fit a SIMD; they live for one memory round trip and a few
 // hundred instructions, so the launch moves through memory as one compact front in the order of
 // the rows instead of as thousands of long-lived streams.  The row is a buffer resource of its
 // own: the lane's vector is the vector offset, the step the instruction's immediate offset (which
