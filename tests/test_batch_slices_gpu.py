@@ -58,12 +58,15 @@ def test_fwd_in_batch_slices(pkg, gpu_device, cc1d_lib, channel_last, seqlen):
 
 
 @pytest.mark.parametrize("overwrite", [0, 1])
+@pytest.mark.parametrize("L", [300, 1100])
 @pytest.mark.parametrize("channel_last", [False, True], ids=["cf", "cl"])
-def test_bwd_in_batch_slices(gpu_device, cc1d_lib, channel_last, overwrite):
+def test_bwd_in_batch_slices(gpu_device, cc1d_lib, channel_last, L, overwrite):
+    """L = 300: channel-first rows of at most 64 vectors (short-row kernel); 1100: tile kernel, three
+    steps a row, one workspace plane per batch entry."""
     lib = cabi.declare(cc1d_lib)
     dev = gpu_device
-    g = gen(57)
-    B, D, L = 9, 136, 300
+    g = gen(57 + L)
+    B, D = 9, 136
     x = make_x(B, D, L, torch.bfloat16, channel_last, g, sliced=False)
     dout = make_x(B, D, L, torch.bfloat16, channel_last, g, sliced=False)
     w, b = make_wb(D, 4, True, g)
@@ -90,9 +93,9 @@ def test_bwd_in_batch_slices(gpu_device, cc1d_lib, channel_last, overwrite):
 
     whole = run(0)
     rdx, rdw, rdb, rdi = orc.bwd(x, w, b, dout, initial_states=init, dfinal_states=dfin, activation="silu")
-    # channel-last: 5120 threads per batch entry (runs of 8 rows), five entries or two to a launch;
-    # channel-first: 136 wavefronts per batch entry, two entries or one to a launch
-    for shift in (16, 17):
+    # L = 300, channel-last: 5120 threads per batch entry (runs of 8 rows), five entries or two to a
+    # launch; channel-first: 136 wavefronts per batch entry, two entries or one to a launch
+    for shift in ((16, 17) if L == 300 else (15, 16)):
         got = run(shift)
         assert torch.equal(got[0], whole[0]) and torch.equal(got[3], whole[3])
         assert_close(got[1], rdw, what="dweight", tol=TOL_W)
