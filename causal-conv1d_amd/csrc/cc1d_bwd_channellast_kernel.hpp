@@ -289,9 +289,11 @@ bwd_channellast_run(const cc1d_bwd_params &p, const BwdClGeom &g, const int32_t 
             for (int j = 0; j < CH; ++j) {
                 dB[j] += gv[j];
 #pragma unroll
+                // a padding row (id < 0) has g = 0; its inputs may hold anything, Inf and NaN
+                // included, and take a zero here so that 0 * x stays 0
                 for (int k = 0; k < W - 1; ++k)
-                    dW[j][k] = fmaf(gv[j], (!MASKED || sqw[k] == cur) ? xw[k][j] : 0.f, dW[j][k]);
-                dW[j][W - 1] = fmaf(gv[j], xv[j], dW[j][W - 1]);
+                    dW[j][k] = fmaf(gv[j], (!MASKED || (sqw[k] == cur && cur >= 0)) ? xw[k][j] : 0.f, dW[j][k]);
+                dW[j][W - 1] = fmaf(gv[j], (!MASKED || cur >= 0) ? xv[j] : 0.f, dW[j][W - 1]);
             }
             dx_row(masked, gw, sqw, gv, cur, dxv);
             if (!decltype(checked)::value) {

@@ -265,8 +265,11 @@ fwd_channellast_kernel(const FwdClArgs a, const FwdClRare q) {
                     for (int j = 0; j < CH; ++j) {
                         float a = bv[j];
 #pragma unroll
+                        // a masked tap takes a zero for its input, not for its weight: what another
+                        // sub-sequence or a padding token holds there (it may be Inf or NaN) must not
+                        // reach this row, as with the reference's conditional add
                         for (int k = 0; k < W - 1; ++k)
-                            a = fmaf(MASKED && ids[u + k] != cur ? 0.f : wv_[j][k], xw[k][j], a);
+                            a = fmaf(wv_[j][k], MASKED && ids[u + k] != cur ? 0.f : xw[k][j], a);
                         a = fmaf(wv_[j][W - 1], xv[j], a);
                         a = SCALED ? silu_from_scaled(a) : SILU ? silu<PRECISE>(a) : a;
                         acc[j] = MASKED && cur < 0 ? 0.f : a;

@@ -172,6 +172,55 @@ def test_fwd_seq_idx_with_sub_sequences_of_a_few_tokens(pkg, gpu_device, dim, se
     assert_close(got, ref, dtype, "out")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seqlen", [40, 517, 2048])
+def test_seq_idx_keeps_non_finite_values_inside_their_sub_sequence(pkg, gpu_device, dtype, seqlen):
+    """Packed sequences are independent requests: Inf or NaN in one of them, or in padding tokens
+    (whose memory may hold anything), must not reach the outputs or gradients of the others.  The
+    reference adds a tap only where the ids agree (csrc/causal_conv1d_fwd.cu:316-329), so nothing
+    is multiplied by a masked input there either."""
+    dev = gpu_device
+    g = gen(4242 + seqlen)
+    B, D, W = 3, 136, 4
+    x = make_x(B, D, seqlen, dtype, True, g, sliced=False)
+    dout = make_x(B, D, seqlen, dtype, True, g, sliced=False)
+    w, b = make_wb(D, W, True, g)
+    third = seqlen // 3
+    seq = torch.zeros(B, seqlen, dtype=torch.int32)
+    seq[:, third:2 * third] = 1
+    seq[:, 2 * third:] = 2
+    seq[:, seqlen - seqlen // 8:] = -1                  # padding tokens
+    poison = torch.tensor([float("nan"), float("inf"), -float("inf")]).to(dtype)
+    dirty_mid, dirty_pad = x.clone(), x.clone()
+    dirty_mid[:, :, third:2 * third] = poison[torch.randint(0, 3, (B, D, 2 * third - third), generator=g)]
+    dirty_pad[:, :, seqlen - seqlen // 8:] = poison[torch.randint(0, 3, (B, D, seqlen // 8), generator=g)]
+    dout_pad = dout.clone()
+    dout_pad[:, :, seqlen - seqlen // 8:] = float("nan")
+    wd, bd, sd = w.to(dev), b.to(dev), seq.to(dev)
+
+    clean = pkg.causal_conv1d_fn(x.to(dev), wd, bd, seq_idx=sd, activation="silu")
+    mid = pkg.causal_conv1d_fn(dirty_mid.to(dev), wd, bd, seq_idx=sd, activation="silu")
+    keep = torch.ones(seqlen, dtype=torch.bool)
+    keep[third:2 * third] = False
+    assert torch.equal(mid[:, :, keep], clean[:, :, keep]), "a poisoned sub-sequence reached its neighbours"
+    assert torch.isfinite(clean).all()
+
+    def fwd_bwd(x_, dout_):
+        xg, wg, bg = x_.to(dev).requires_grad_(), wd.clone().requires_grad_(), bd.clone().requires_grad_()
+        out = pkg.causal_conv1d_fn(xg, wg, bg, seq_idx=sd, activation="silu")
+        out.backward(dout_.to(dev))
+        return out.detach(), xg.grad, wg.grad, bg.grad
+
+    ref = fwd_bwd(x, dout)
+    got = fwd_bwd(dirty_pad, dout_pad)
+    valid = (seq[0] >= 0)
+    assert torch.equal(got[0], ref[0]), "padding tokens reached the outputs"
+    assert bool((got[0][:, :, ~valid] == 0).all())
+    assert torch.equal(got[1][:, :, valid], ref[1][:, :, valid]), "padding tokens reached dx"
+    assert bool((got[1][:, :, ~valid] == 0).all()), "dx of padding tokens is zero"
+    assert torch.equal(got[2], ref[2]) and torch.equal(got[3], ref[3]), "padding tokens reached dweight / dbias"
+
+
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("channel_last", [False, True])
