@@ -95,6 +95,52 @@ bool states_overlap(const cc1d_fwd_params &p) {
     return false;
 }
 
+// Do an input and an output of shape (batch, dim, seqlen) provably share an element?  No kernel
+// here works in place: a row's halo is read by another wavefront than the one that writes the
+// positions in front of it.  Decided only where it can be decided exactly -- the same strides for
+// both views, nested (each stride larger than everything the smaller ones span): the views then
+// share an element iff the distance between their bases is a sum of in-range index differences,
+// and with nested strides each difference has two candidates at most.  Anything else (different
+// strides, byte ranges that merely interleave, as two column slices of one wider buffer do) is
+// let through, as the reference lets everything through.
+bool views_share_an_element(int batch, int dim, int seqlen, int eb, const void *a, const void *b, int64_t sb,
+                            int64_t sc, int64_t sl, int64_t sb2, int64_t sc2, int64_t sl2) {
+    if (a == nullptr || b == nullptr) return false;
+    int64_t n[3] = {batch, dim, seqlen}, st[3] = {sb, sc, sl}, st2[3] = {sb2, sc2, sl2};
+    for (int i = 0; i < 3; ++i)
+        if (n[i] > 1 && (st[i] != st2[i] || st[i] <= 0)) return false;
+    const int64_t bytes = (int64_t)(reinterpret_cast<uintptr_t>(b) - reinterpret_cast<uintptr_t>(a));
+    if (bytes % eb != 0) return false;
+    // dimensions that matter, by falling stride
+    int order[3], m = 0;
+    for (int i = 0; i < 3; ++i)
+        if (n[i] > 1) order[m++] = i;
+    for (int i = 0; i < m; ++i)
+        for (int j = i + 1; j < m; ++j)
+            if (st[order[j]] > st[order[i]]) { const int t = order[i]; order[i] = order[j]; order[j] = t; }
+    int64_t inner[3];                                  // what the dimensions behind i span
+    for (int i = m - 1; i >= 0; --i) {
+        inner[i] = i == m - 1 ? 0 : inner[i + 1] + (n[order[i + 1]] - 1) * st[order[i + 1]];
+        if (st[order[i]] <= inner[i]) return false;   // not nested: undecided
+    }
+    // depth-first over the candidates: |rest - d * stride| must not exceed what is left behind
+    struct Walk {
+        const int64_t *n, *st, *inner; const int *order; int m;
+        bool operator()(int i, int64_t rest) const {
+            if (i == m) return rest == 0;
+            const int64_t s = st[order[i]];
+            int64_t d = rest / s;
+            if (rest % s != 0 && rest < 0) --d;        // floor
+            for (int64_t c = d; c <= d + 1; ++c) {
+                const int64_t r = rest - c * s;
+                if (c > -n[order[i]] && c < n[order[i]] && r >= -inner[i] && r <= inner[i] && (*this)(i + 1, r)) return true;
+            }
+            return false;
+        }
+    };
+    return Walk{n, st, inner, order, m}(0, bytes / eb);
+}
+
 // ---- batch slicing ---------------------------------------------------------------------------
 // A launcher refuses, before launching anything, a problem that needs more work items than one
 // grid holds (CC1D_ERR_TOO_LARGE).  Every batch entry is independent, so the front then halves
@@ -231,6 +277,7 @@ const char *cc1d_strerror(int status) {
         case CC1D_ERR_LAUNCH: return "HIP kernel launch failed";
         case CC1D_ERR_UNKNOWN_TUNABLE: return "unknown tunable name";
         case CC1D_ERR_WORKSPACE_LIMIT: return "backward needs more workspace than the library's built-in array holds; use cc1d_bwd with a caller-owned workspace";
+        case CC1D_ERR_IN_PLACE: return "an output shares elements with an input (out with x, dx with x or dout): the kernels do not work in place";
         default: return "unknown cc1d status";
     }
 }
@@ -296,6 +343,9 @@ int cc1d_validate_fwd(const cc1d_fwd_params *p) {
                            p->out_stride_c, p->out_stride_l);
     if (st != CC1D_OK) return st;
     if (p->seq_idx != nullptr && !cl) return CC1D_ERR_SEQ_IDX_LAYOUT;
+    if (views_share_an_element(p->batch, p->dim, p->seqlen, elem_bytes(p->x_dtype), p->x, p->out, p->x_stride_b,
+                               p->x_stride_c, p->x_stride_l, p->out_stride_b, p->out_stride_c, p->out_stride_l))
+        return CC1D_ERR_IN_PLACE;
     // initial_states and final_states may be one and the same tensor (csrc/causal_conv1d.h:44 of the
     // reference: a chunked prefill that keeps a single state buffer): same address, same strides.
     // Every kernel reads a row's initial_states and writes its final_states from one wavefront, reads
@@ -359,6 +409,12 @@ int cc1d_validate_bwd(const cc1d_bwd_params *p) {
     st = check_same_family(cl, p->x_dtype, p->batch, p->seqlen, p->dx, p->dx_stride_b,
                            p->dx_stride_c, p->dx_stride_l);
     if (st != CC1D_OK) return st;
+    const int eb = elem_bytes(p->x_dtype);
+    if (views_share_an_element(p->batch, p->dim, p->seqlen, eb, p->x, p->dx, p->x_stride_b, p->x_stride_c, p->x_stride_l,
+                               p->dx_stride_b, p->dx_stride_c, p->dx_stride_l) ||
+        views_share_an_element(p->batch, p->dim, p->seqlen, eb, p->dout, p->dx, p->dout_stride_b, p->dout_stride_c,
+                               p->dout_stride_l, p->dx_stride_b, p->dx_stride_c, p->dx_stride_l))
+        return CC1D_ERR_IN_PLACE;
     if (p->seq_idx != nullptr) {
         if (!cl) return CC1D_ERR_SEQ_IDX_LAYOUT;
         if (p->initial_states != nullptr || p->dfinal_states != nullptr || p->dinitial_states != nullptr)

@@ -59,7 +59,8 @@ typedef enum cc1d_status {
     CC1D_ERR_TOO_LARGE = -16,        /* one batch entry alone exceeds what a grid can express */
     CC1D_ERR_LAUNCH = -17,           /* the HIP runtime refused the launch */
     CC1D_ERR_UNKNOWN_TUNABLE = -18,
-    CC1D_ERR_WORKSPACE_LIMIT = -19   /* cc1d_bwd_noalloc: the problem needs more than the built-in workspace */
+    CC1D_ERR_WORKSPACE_LIMIT = -19,  /* cc1d_bwd_noalloc: the problem needs more than the built-in workspace */
+    CC1D_ERR_IN_PLACE = -20          /* out shares elements with x, or dx with x or dout: no kernel works in place */
 } cc1d_status;
 
 /* Opaque stream handle: pass a hipStream_t (NULL = the default stream). */

@@ -136,6 +136,41 @@ def test_validate_fwd_states_that_share_memory(lib):
     assert v(p) == E_STATE_LAYOUT                       # same bytes under two different views
 
 
+def test_outputs_that_share_elements_with_inputs_are_refused(lib):
+    """No kernel works in place (a row's halo is read by another wavefront than the one that
+    writes the positions in front of it).  Refused only where a shared element is certain: the
+    same nested strides for both views.  Views that merely interleave in memory pass."""
+    E_IN_PLACE = -20
+    B, D, L, W = 2, 16, 24, 4
+    w, b = torch.zeros(D, W), torch.zeros(D)
+
+    def fwd(x, out):
+        return lib.cc1d_validate_fwd(cabi.fwd_params(x, w, b, out, True))
+
+    for channel_last in (False, True):
+        wide = torch.zeros(B, L, 3 * D).transpose(1, 2) if channel_last else torch.zeros(B, 3 * D, L)
+        x = wide[:, 0:D, :]
+        assert fwd(x, x) == E_IN_PLACE                             # in place
+        assert fwd(x, wide[:, D:2 * D, :]) == OK                   # a neighbouring slice of the same buffer
+        assert fwd(x, wide[:, D // 2:D // 2 + D, :]) == E_IN_PLACE  # half of the channels in common
+        assert fwd(wide[:, D:2 * D, :], x) == OK
+        assert fwd(wide[:, D // 2:D // 2 + D, :], x) == E_IN_PLACE
+        long_ = torch.zeros(B, 2 * L + 8, D).transpose(1, 2) if channel_last else torch.zeros(B, D, 2 * L + 8)
+        assert fwd(long_[:, :, 0:L], long_[:, :, L:2 * L]) == OK   # two windows along seqlen
+        assert fwd(long_[:, :, 0:L], long_[:, :, L - 1:2 * L - 1]) == E_IN_PLACE
+        assert fwd(long_[:, :, 8:L + 8], long_[:, :, 0:L]) == E_IN_PLACE
+        fresh = torch.zeros_like(wide)[:, 0:D, :]
+        assert fwd(x, fresh) == OK
+    p, _k = _bwd(channel_last=True)
+    assert lib.cc1d_validate_bwd(p) == OK
+    p.dx, p.dx_stride_b, p.dx_stride_c, p.dx_stride_l = p.dout, p.dout_stride_b, p.dout_stride_c, p.dout_stride_l
+    assert lib.cc1d_validate_bwd(p) == E_IN_PLACE                  # dx written over dout
+    p, _k = _bwd(channel_last=False)
+    p.dx, p.dx_stride_b, p.dx_stride_c, p.dx_stride_l = p.x, p.x_stride_b, p.x_stride_c, p.x_stride_l
+    assert lib.cc1d_validate_bwd(p) == E_IN_PLACE                  # dx written over x
+    assert b"in place" in lib.cc1d_strerror(E_IN_PLACE)
+
+
 def _bwd(channel_last=False, bias=True):
     B, D, L, W = 2, 16, 24, 4
     mk = (lambda: torch.zeros(B, L, D).transpose(1, 2)) if channel_last else (lambda: torch.zeros(B, D, L))
