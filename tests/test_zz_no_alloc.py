@@ -97,12 +97,13 @@ def test_no_alloc_backward_refuses_what_does_not_fit(cc1d_lib):
     B, D, L = 16, 5376, 2048
     class Shaped:                                       # a tensor's shape, strides and address, no storage
         dtype, shape = torch.bfloat16, (B, D, L)
+        def __init__(self, nth): self.nth = nth
         def stride(self, ax): return (L * D, 1, D)[ax]  # channel-last
-        def data_ptr(self): return 1 << 20              # any 16-byte aligned non-NULL address
-    x = Shaped()
+        def data_ptr(self): return (1 + self.nth) << 30 # 16-byte aligned, non-NULL, one GiB apart
+    x, dout, dx = Shaped(0), Shaped(1), Shaped(2)
     w, b = torch.zeros(D, 4), torch.zeros(D)
     dw, db = torch.zeros(D, 4), torch.zeros(D)
-    p = cabi.bwd_params(x, w, b, x, x, dw, db, True)
+    p = cabi.bwd_params(x, w, b, dout, dx, dw, db, True)
     need = ctypes.c_size_t()
     assert lib.cc1d_bwd_workspace_bytes(ctypes.byref(p), ctypes.byref(need)) == 0
     assert need.value > MAX_WS
