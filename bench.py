@@ -19,7 +19,8 @@ Prints ONE JSON line.  A "step" is one forward call at the Mamba-2 2.7B prefill 
                      (a few milliseconds of load at the highest clock); `frac_rotated` runs over
                      six rotating sets of x and out (2.1 GB), where no launch finds its tensors in
                      a cache, as the layers of a model do, behind the same 400 untimed launches
-                     (none with --no-settle).  `decode` repeats
+                     (none with --no-settle); config.us_per_call_rotated_12_sets is the same over
+                     twelve sets (4.2 GB).  `decode` repeats
                      the three figures for the two decode-step updates.  `traffic` is imported
                      from the committed rocprofv3 summary, not measured in this run
   cpu_baseline ..... the PyTorch oracle (F.conv1d per packed sub-sequence) timed on this
@@ -529,6 +530,14 @@ def main():
                                "GBps_rotated": round(gbs(n_bytes, rot_us), 1),
                                "us_torch_add_rotated": round(add_us, 3)})
         line["roofline"]["frac_rotated"] = round(gbs(n_bytes, rot_us) / HBM_PEAK_GBS, 4)
+        # Twelve sets (4.2 GB): past the reach of the address-translation caches as well, which a
+        # kernel that walks rows a row stride apart feels and a linear sweep does not.
+        sets += [(torch.randn_like(x), torch.empty_like(x)) for _ in range(6)]
+        rot12_us, _ = time_gpu(lambda i: ext.causal_conv1d_fwd(sets[i % 12][0], w, b, seq, None, sets[i % 12][1], None, True),
+                               args.steps, args.warmup + settle)
+        add12_us, _ = time_gpu(lambda i: torch.add(sets[i % 12][0], 1.0, out=sets[i % 12][1]), args.steps, args.warmup + settle)
+        line["config"].update({"us_per_call_rotated_12_sets": round(rot12_us, 3),
+                               "us_torch_add_rotated_12_sets": round(add12_us, 3)})
         del sets
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(cfg_cpu, n_bytes, gpu_out_host)
