@@ -108,7 +108,7 @@ def _segments(row):
 def test_every_update_combination(pkg, gpu_device, dtype):
     """The reference's three decode-step grids in full (tests/test_causal_conv1d.py:140-321):
     dim x width x seqlen x cache_seqlens x bias x SiLU, each combination plain, through
-    conv_state_indices into a ten times larger cache, and with half the requests padding
+    conv_state_indices into a larger cache, and with half the requests padding
     (index -1; the reference runs that one without cache_seqlens, here both).  648 cases per
     dtype; conv_state bit-exact, untouched rows untouched, padded outputs exactly zero."""
     dev = gpu_device
@@ -122,7 +122,7 @@ def test_every_update_combination(pkg, gpu_device, dtype):
             g = gen(n * 7 + dim)
             x = torch.randn(batch, seqlen, dim, generator=g).to(dtype).transpose(-1, -2)
             state_len = int(torch.randint(width - 1, width + 10, (1,), generator=g))
-            entries = batch if variant == "plain" else 10 * batch
+            entries = batch if variant == "plain" else 3 * batch    # (ten times in the reference: test_update_gpu.py keeps that)
             st = torch.randn(entries, state_len, dim, generator=g).to(dtype).transpose(-1, -2)
             w, b = make_wb(dim, width, has_bias, g)
             cs = torch.randint(0, 1024, (batch,), generator=g, dtype=torch.int32) if circular else None
