@@ -35,6 +35,7 @@ namespace {
 constexpr int kTileSteps = 4;                     // 64-vector steps per tile
 constexpr int kTileVecs = kTileSteps * kWave;     // 256 vectors, 4 KiB
 constexpr int kTailVecs = kWave / 4;              // most vectors 64 positions can span (fp32)
+constexpr int kLdsVecs = kTileVecs + 1 + kTailVecs; // LDS vectors of one wavefront
 constexpr int kRsrcRaw = 0x00020000;              // buffer resource word 3: raw buffer, 32-bit data format
 
 typedef void __attribute__((address_space(3))) *lds_ptr_t;
@@ -70,7 +71,7 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
     constexpr int EB = E::kBytes;
     constexpr bool PRECISE = E::kPreciseAct;
     constexpr bool SCALED = SILU && !PRECISE;         // taps and bias carry the factor of the SiLU exponent
-    __shared__ u32x4 lds[kBlock / kWave][kTileVecs + 1 + kTailVecs];   // [wavefront][halo vector + tile + tail]
+    extern __shared__ u32x4 lds[];                    // [wavefront][halo vector + tile + tail]
 
     const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     const int lane = (int)(threadIdx.x & (kWave - 1));
@@ -105,7 +106,7 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
     // LDS vector i of the wavefront holds row vector v0 - 1 + i.  For the row's first tile the
     // offset below wraps around: out of range, LDS gets zeros (the row's zero padding).
     const int vx = (lane + v0 - 1) * 16;
-    u32x4 *mine = &lds[wv][0];
+    u32x4 *mine = lds + wv * kLdsVecs;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 0, 2);
     if (steps > 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 1024, 2);
     if (steps > 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)mine, 16, vx, 0, 2048, 2);
@@ -202,8 +203,15 @@ fwd_channelfirst_tile_kernel(const FwdCfTileArgs a) {
 template <int DT, int W>
 int launch_tile_act(const cc1d_fwd_params &p, const FwdCfTileArgs &a, hipStream_t stream) {
     const uint32_t blocks = (a.total + (kBlock / kWave) - 1) / (kBlock / kWave);
-    if (p.silu) CC1D_LAUNCH((fwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), 0, stream, a);
-    else CC1D_LAUNCH((fwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), 0, stream, a);
+    // What the four wavefronts' tiles take (eight workgroups fit a CU), and for rows of three steps
+    // and more a fifth of a CU's LDS: wavefronts that fetch 3-4 KiB each run 2-4 % faster five
+    // workgroups to a CU than eight -- (8, 5376, 2048) bf16 57.9 -> 56.6 us, (4, 4096, 8192) fp16
+    // 87.6 -> 83.8, (8, 5376, 4095) 123.5 -> 120.9 -- while rows of two steps lose ((16, 4096, 1001)
+    // 48.6 -> 56.0 us) and keep all eight.
+    size_t lds = (size_t)(kBlock / kWave) * kLdsVecs * sizeof(u32x4);
+    if (a.body_vecs > 2 * kWave && lds < 160 * 1024 / 5) lds = 160 * 1024 / 5;
+    if (p.silu) CC1D_LAUNCH((fwd_channelfirst_tile_kernel<DT, W, true>), dim3(blocks), dim3(kBlock), lds, stream, a);
+    else CC1D_LAUNCH((fwd_channelfirst_tile_kernel<DT, W, false>), dim3(blocks), dim3(kBlock), lds, stream, a);
     return launch_status();
 }
 
